@@ -1,0 +1,199 @@
+// C ABI of libbsa_hip.so: argument validation and dispatch (see include/bsa.h).
+// Takes over what the reference does in sparse/native/sparse_kernels.cc:39-46
+// (dtype switch) and in its kernel wrappers (sparse_smm_gpu.cu:270-293), and
+// adds the checks the reference lacks: every size the kernels index with is
+// validated on the host before a launch.
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/bsa.h"
+#include "bsa_internal.hpp"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(hipError_t err, const char *what)
+{
+    if (err == hipSuccess) return BSA_OK;
+    return fail(BSA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(err));
+}
+
+constexpr int MAX_WAVES = 8;
+constexpr long long MAX_GRID = 2147483647LL;
+
+int check_schedule(const int32_t *sched, int sched_wgs, int sched_waves, int batches, const char *who)
+{
+    if (!sched) return fail(BSA_ERR_INVALID, "%s: schedule is null", who);
+    if (sched_waves < 1 || sched_waves > MAX_WAVES)
+        return fail(BSA_ERR_INVALID, "%s: schedule waves per workgroup %d outside [1, %d]", who, sched_waves, MAX_WAVES);
+    if (sched_wgs < 1) return fail(BSA_ERR_INVALID, "%s: schedule has %d workgroups", who, sched_wgs);
+    if (8LL * sched_wgs * ((batches + 7) / 8) > MAX_GRID)
+        return fail(BSA_ERR_INVALID, "%s: grid of %d workgroups x %d batches is too large", who, sched_wgs, batches);
+    return BSA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int bsa_version(void) { return 100; }
+
+const char *bsa_last_error(void) { return g_error; }
+
+size_t bsa_layout_workspace_bytes(int mask_rows, int mask_cols)
+{
+    if (mask_rows < 1 || mask_cols < 1) return 0;
+    return (size_t)mask_rows * (size_t)mask_cols * sizeof(int32_t);
+}
+
+int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
+                     int32_t *row_blocks, int32_t *row_offsets,
+                     int32_t *col_blocks, int32_t *col_offsets,
+                     int32_t *nnz_out, void *workspace, void *stream)
+{
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "bsa_layout_build: mask shape %d x %d outside [1, 32767] x [1, 65535]",
+                    mask_rows, mask_cols);
+    if ((long long)mask_rows * mask_cols > (1LL << 28))
+        return fail(BSA_ERR_INVALID, "bsa_layout_build: mask of %d x %d cells is too large", mask_rows, mask_cols);
+    if (!mask || !row_blocks || !row_offsets || !col_blocks || !col_offsets || !nnz_out || !workspace)
+        return fail(BSA_ERR_INVALID, "bsa_layout_build: null pointer argument");
+    return check_launch(bsa::launch_layout_build(mask, mask_rows, mask_cols, row_blocks, row_offsets,
+                                                 col_blocks, col_offsets, nnz_out, workspace,
+                                                 (hipStream_t)stream),
+                        "bsa_layout_build");
+}
+
+int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves)
+{
+    if (groups < 1 || nnz < 0 || cap < 1 || waves < 1) return 0;
+    int64_t slots = 2 * ((int64_t)groups + nnz / cap + 1) + waves;
+    return slots + (groups + 3) / 4;
+}
+
+int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
+                       int32_t *sched, int64_t capacity, int32_t *n_wgs_out, void *stream)
+{
+    if (!offsets || !sched || !n_wgs_out) return fail(BSA_ERR_INVALID, "bsa_schedule_build: null pointer argument");
+    if (groups < 1 || groups > 65535) return fail(BSA_ERR_INVALID, "bsa_schedule_build: %d groups outside [1, 65535]", groups);
+    if (cap < 1) return fail(BSA_ERR_INVALID, "bsa_schedule_build: cap %d < 1", cap);
+    if (waves < 1 || waves > MAX_WAVES)
+        return fail(BSA_ERR_INVALID, "bsa_schedule_build: waves %d outside [1, %d]", waves, MAX_WAVES);
+    if (capacity < 2 * ((int64_t)groups + 1) + waves + (groups + 3) / 4 || capacity > (1LL << 28))
+        return fail(BSA_ERR_INVALID, "bsa_schedule_build: capacity %lld too small for %d groups (use bsa_schedule_capacity)",
+                    (long long)capacity, groups);
+    return check_launch(bsa::launch_schedule_build(offsets, groups, cap, waves, sched, capacity, n_wgs_out,
+                                                   (hipStream_t)stream),
+                        "bsa_schedule_build");
+}
+
+int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
+               const int32_t *blocks, const int32_t *offsets, int groups,
+               const int32_t *sched, int sched_wgs, int sched_waves,
+               int mask_rows, int mask_cols, int nnz, int batches,
+               int M, int N, int K, int tr_a, int tr_b, void *stream)
+{
+    if (mode != BSA_SDD && mode != BSA_DSD && mode != BSA_DDS)
+        return fail(BSA_ERR_INVALID, "bsa_matmul: unknown mode %d", mode);
+    if (dtype != BSA_F32 && dtype != BSA_F16)
+        return fail(BSA_ERR_UNSUPPORTED, "bsa_matmul: unsupported dtype %d (fp32 = 0, fp16 = 1)", dtype);
+    // with nnz == 0 the table and the sparse tensor are empty and may be null
+    const bool a_needed = nnz > 0 || mode != BSA_DSD, b_needed = nnz > 0 || mode != BSA_DDS;
+    const bool c_needed = nnz > 0 || mode != BSA_SDD;
+    if ((!a && a_needed) || (!b && b_needed) || (!c && c_needed) || (!blocks && nnz > 0) || !offsets)
+        return fail(BSA_ERR_INVALID, "bsa_matmul: null pointer argument");
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "bsa_matmul: mask shape %d x %d out of range", mask_rows, mask_cols);
+    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
+        return fail(BSA_ERR_INVALID, "bsa_matmul: nnz %d does not fit a %d x %d mask", nnz, mask_rows, mask_cols);
+    if (batches < 1) return fail(BSA_ERR_INVALID, "bsa_matmul: batches %d < 1", batches);
+    if (M < 1 || N < 1 || K < 1 || M % BSA_BLOCK || N % BSA_BLOCK || K % BSA_BLOCK)
+        return fail(BSA_ERR_INVALID, "bsa_matmul: M, N, K = %d, %d, %d must be positive multiples of %d", M, N, K, BSA_BLOCK);
+    int rc = check_schedule(sched, sched_wgs, sched_waves, batches, "bsa_matmul");
+    if (rc) return rc;
+
+    // which table the caller must have passed, and what the sparse matrix spans
+    const bool row_table = mode == BSA_SDD || (mode == BSA_DSD && !tr_a) || (mode == BSA_DDS && tr_b);
+    const int want_groups = row_table ? mask_rows : mask_cols;
+    if (groups != want_groups)
+        return fail(BSA_ERR_INVALID, "bsa_matmul: table has %d groups, the %s layout of a %d x %d mask has %d",
+                    groups, row_table ? "row" : "column", mask_rows, mask_cols, want_groups);
+    const int SR = BSA_BLOCK * mask_rows, SC = BSA_BLOCK * mask_cols;
+    if (mode == BSA_SDD) {
+        if (M != SR || N != SC)
+            return fail(BSA_ERR_INVALID, "bsa_matmul sdd: op(a) has %d rows and op(b) %d columns, the layout spans %d x %d",
+                        M, N, SR, SC);
+    } else if (mode == BSA_DSD) {
+        const int m_want = tr_a ? SC : SR, k_want = tr_a ? SR : SC;
+        if (M != m_want || K != k_want)
+            return fail(BSA_ERR_INVALID, "bsa_matmul dsd: M, K = %d, %d but op(sparse a) is %d x %d", M, K, m_want, k_want);
+    } else {
+        const int k_want = tr_b ? SC : SR, n_want = tr_b ? SR : SC;
+        if (K != k_want || N != n_want)
+            return fail(BSA_ERR_INVALID, "bsa_matmul dds: K, N = %d, %d but op(sparse b) is %d x %d", K, N, k_want, n_want);
+    }
+    const int free_dim = mode == BSA_SDD ? K : (mode == BSA_DSD ? N : M);
+    if ((free_dim + 63) / 64 > 65535)
+        return fail(BSA_ERR_INVALID, "bsa_matmul: dense dimension %d is too large", free_dim);
+
+    bsa::MatmulArgs p{a, b, c, blocks, sched, sched_wgs, sched_waves, nnz, batches, M, N, K, tr_a != 0, tr_b != 0};
+    if (nnz == 0 && mode == BSA_SDD) return BSA_OK;   // nothing to write
+    hipError_t err = mode == BSA_SDD ? bsa::launch_sdd(dtype, p, (hipStream_t)stream)
+                                     : bsa::launch_group_walk(dtype, mode == BSA_DSD, p, (hipStream_t)stream);
+    return check_launch(err, "bsa_matmul");
+}
+
+static int check_softmax(const char *who, int dtype, const void *p0, const void *p1, const void *p2,
+                         const int32_t *blocks, const int32_t *offsets, const int32_t *sched,
+                         int sched_wgs, int sched_waves, int mask_rows, int mask_cols, int nnz, int batches)
+{
+    if (dtype != BSA_F32 && dtype != BSA_F16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: unsupported dtype %d (fp32 = 0, fp16 = 1)", who, dtype);
+    if (!p0 || !p1 || !p2 || !blocks || !offsets) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
+    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
+        return fail(BSA_ERR_INVALID, "%s: nnz %d does not fit a %d x %d mask", who, nnz, mask_rows, mask_cols);
+    if (batches < 1) return fail(BSA_ERR_INVALID, "%s: batches %d < 1", who, batches);
+    return check_schedule(sched, sched_wgs, sched_waves, batches, who);
+}
+
+int bsa_softmax_forward(int dtype, const void *x, void *y,
+                        const int32_t *row_blocks, const int32_t *row_offsets,
+                        const int32_t *sched, int sched_wgs, int sched_waves,
+                        int mask_rows, int mask_cols, int nnz, int batches,
+                        float scale, int causal, void *stream)
+{
+    int rc = check_softmax("bsa_softmax_forward", dtype, x, y, y, row_blocks, row_offsets, sched, sched_wgs,
+                           sched_waves, mask_rows, mask_cols, nnz, batches);
+    if (rc) return rc;
+    if (nnz == 0) return BSA_OK;
+    bsa::SoftmaxArgs p{x, nullptr, y, row_blocks, sched, sched_wgs, sched_waves, nnz, batches, scale, causal != 0};
+    return check_launch(bsa::launch_softmax_forward(dtype, p, (hipStream_t)stream), "bsa_softmax_forward");
+}
+
+int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
+                         const int32_t *row_blocks, const int32_t *row_offsets,
+                         const int32_t *sched, int sched_wgs, int sched_waves,
+                         int mask_rows, int mask_cols, int nnz, int batches,
+                         float scale, void *stream)
+{
+    int rc = check_softmax("bsa_softmax_backward", dtype, y, dy, dx, row_blocks, row_offsets, sched, sched_wgs,
+                           sched_waves, mask_rows, mask_cols, nnz, batches);
+    if (rc) return rc;
+    if (nnz == 0) return BSA_OK;
+    bsa::SoftmaxArgs p{y, dy, dx, row_blocks, sched, sched_wgs, sched_waves, nnz, batches, scale, false};
+    return check_launch(bsa::launch_softmax_backward(dtype, p, (hipStream_t)stream), "bsa_softmax_backward");
+}
+
+}  // extern "C"

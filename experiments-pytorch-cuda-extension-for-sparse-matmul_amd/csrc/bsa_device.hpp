@@ -1,0 +1,139 @@
+// Device-side building blocks shared by the gfx950 kernels: table decode,
+// MFMA fragments, the wave-private LDS transpose and the workgroup -> (batch,
+// schedule slot) mapping.  gfx950 only: 64-wide wavefronts, v_mfma_f32_32x32x16_f16,
+// v_mfma_f32_32x32x2_f32, ds_read_b64_tr_b16.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bsa {
+
+typedef _Float16 half_t;
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef __fp16 tr4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+
+constexpr int BS = 32;          // block edge
+constexpr int BS2 = BS * BS;    // elements per block
+constexpr int WAVE = 64;
+
+// One pair of the block table (sparse/native/sparse_layout.cuh:13-21 keeps the
+// same two ints; the column is decoded from 16 bits here, not 8).
+struct BlockDesc {
+    int idx;
+    int pos;
+    __device__ __forceinline__ int row() const { return (int)((unsigned)pos >> 16); }
+    __device__ __forceinline__ int col() const { return pos & 0xFFFF; }
+};
+
+// One wavefront slot of a schedule.
+struct SchedEntry {
+    int group;   // -1: unused slot
+    int begin;   // first pair of the chunk
+    int end;     // one past the last pair
+    int team;    // (slot of the team's first wave in the workgroup) | (team waves << 8)
+};
+
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63u); }
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
+// MFMA 32x32 accumulators give lane (l % 32, h = l / 32) the result rows
+// 8 * (v / 4) + 4 * h + v % 4, v = 0..15.  Feeding the row operand through this
+// permutation makes those 16 values 16 CONSECUTIVE logical indices 16 * h + v,
+// so a lane can store them with two 16-byte (fp16) or four (fp32) writes.
+__device__ __forceinline__ int perm16(int i) { return (i & 3) + 4 * (i >> 3) + 16 * ((i >> 2) & 1); }
+
+// Workgroup -> (batch, schedule workgroup).  Hardware deals consecutive
+// workgroup ids round-robin to the 8 XCDs, each with its own 4 MB L2; batch b
+// is pinned to XCD b % 8 so that its dense operand is fetched into one L2 only.
+// The grid holds 8 * n_swg * ceil(batches / 8) workgroups.
+__device__ __forceinline__ bool map_workgroup(int n_swg, int batches, int &batch, int &swg)
+{
+    int w = (int)blockIdx.x;
+    int t = w >> 3;
+    batch = (w & 7) + 8 * (t / n_swg);
+    swg = t % n_swg;
+    return batch < batches;
+}
+
+// Orders the LDS traffic of ONE wavefront: what its lanes wrote before is
+// visible to all its lanes after.  LDS executes a wave's instructions in
+// order, so this only has to stop the compiler from moving accesses across.
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ds_read_b64_tr_b16: inside every group of 16 lanes, source lane s hands in
+// the address of 4 consecutive halves; result lane i receives, as element e,
+// element (i % 4) of source lane 4 * e + i / 4.  With source lane s pointing at
+// row s / 4, column chunk s % 4 of a [k][x] tile, result lane 4 * a + c holds
+// k = 0..3 of column chunk(a) + c: the MFMA operand layout out of a tile whose
+// contraction index is the slow one.
+__device__ __forceinline__ h4 lds_read_tr16(const half_t *p)
+{
+    typedef tr4 __attribute__((address_space(3))) *lds_tr4_ptr;
+    tr4 r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_tr4_ptr)(uintptr_t)p);
+    return __builtin_bit_cast(h4, r);
+}
+
+// Chunk base (in elements) handed in by source lane quad a = s % 4 of lane
+// group g = lane / 16, for a 32-wide index range: natural order gives result
+// lane l the index l % 32; the permuted order gives it perm16(l % 32).
+template <bool PERMUTED>
+__device__ __forceinline__ int tr_chunk_base(int g, int a)
+{
+    if (PERMUTED) return 8 * (g & 1) + 4 * (a >> 1) + 16 * (a & 1);
+    return 16 * (g & 1) + 4 * a;
+}
+
+// Reads the 8 halves k = 16 * step + 8 * (lane / 32) + 0..7 of one index from a
+// [k][x] tile in LDS with row stride `ld` halves; `x0` is the first column of
+// the 32-wide index range.
+template <bool PERMUTED>
+__device__ __forceinline__ h8 lds_operand_tr(const half_t *tile, int ld, int x0, int step)
+{
+    int l = lane_id();
+    int g = l >> 4, s = l & 15;
+    int k = 16 * step + 8 * (g >> 1) + (s >> 2);
+    int x = x0 + tr_chunk_base<PERMUTED>(g, s & 3);
+    h4 lo = lds_read_tr16(tile + k * ld + x);
+    h4 hi = lds_read_tr16(tile + (k + 4) * ld + x);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+__device__ __forceinline__ f16v mfma_f16(h8 a, h8 b, f16v c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f16v mfma_f32(float a, float b, f16v c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint4 ldg16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
+__device__ __forceinline__ void stg16(void *p, uint4 v) { *reinterpret_cast<uint4 *>(p) = v; }
+
+__device__ __forceinline__ h8 as_h8(uint4 v) { return __builtin_bit_cast(h8, v); }
+
+// 16 fp32 accumulators -> 16 halves in two 16-byte registers.
+__device__ __forceinline__ void pack16(const f16v &acc, uint4 &lo, uint4 &hi)
+{
+    h8 a, b;
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+        a[v] = (half_t)acc[v];
+        b[v] = (half_t)acc[v + 8];
+    }
+    lo = __builtin_bit_cast(uint4, a);
+    hi = __builtin_bit_cast(uint4, b);
+}
+
+}  // namespace bsa

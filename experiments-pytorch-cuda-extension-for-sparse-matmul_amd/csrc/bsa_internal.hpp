@@ -1,0 +1,47 @@
+// Host-side launchers behind the C ABI (one per kernel family).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bsa {
+
+hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_blocks,
+                               int32_t *row_off, int32_t *col_blocks, int32_t *col_off,
+                               int32_t *nnz_out, void *workspace, hipStream_t stream);
+
+hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
+                                 int32_t *sched, int64_t capacity, int32_t *n_wgs_out,
+                                 hipStream_t stream);
+
+struct MatmulArgs {
+    const void *a, *b;
+    void *c;
+    const int32_t *blocks;
+    const int32_t *sched;
+    int sched_wgs, sched_waves;
+    int nnz, batches;
+    int M, N, K;
+    bool tr_a, tr_b;
+};
+
+hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t stream);
+// group walk shared by DSD (dsd = true) and DDS
+hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream_t stream);
+
+struct SoftmaxArgs {
+    const void *x;    // forward: scores; backward: y
+    const void *dy;   // backward only
+    void *out;
+    const int32_t *blocks;
+    const int32_t *sched;
+    int sched_wgs, sched_waves;
+    int nnz, batches;
+    float scale;
+    bool causal;
+};
+
+hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t stream);
+hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t stream);
+
+}  // namespace bsa

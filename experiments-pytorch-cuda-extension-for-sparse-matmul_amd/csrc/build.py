@@ -1,0 +1,47 @@
+"""Builds libbsa_hip.so for gfx950 with hipcc (no torch headers, no cmake).
+
+    python build.py            # rebuild when a source is newer than the library
+    python build.py --force    # always rebuild
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SOURCES = ["api.hip", "layout_build.hip", "matmul.hip", "softmax.hip"]
+HEADERS = ["bsa_device.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
+LIB = os.path.join(HERE, "libbsa_hip.so")
+
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-fno-gpu-rdc", "-Wall", "-Wno-unused-function",
+    # keep the compiler from forming packed-fp32 instructions out of scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def out_of_date() -> bool:
+    if not os.path.exists(LIB):
+        return True
+    t = os.path.getmtime(LIB)
+    return any(os.path.getmtime(os.path.join(HERE, f)) > t for f in SOURCES + HEADERS + ["build.py"])
+
+
+def build(force: bool = False, verbose: bool = False) -> str:
+    if not force and not out_of_date():
+        return LIB
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + FLAGS + [os.path.join(HERE, s) for s in SOURCES] + ["-o", LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("hipcc failed building libbsa_hip.so")
+    if verbose and res.stderr.strip():
+        sys.stderr.write(res.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv, verbose=True))

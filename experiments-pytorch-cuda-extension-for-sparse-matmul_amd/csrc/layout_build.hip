@@ -1,0 +1,158 @@
+// Device-side builder of the block-index tables and of the wavefront schedule.
+//
+// Tables: the contract is the output of SparseLayout._create_layout
+// (sparse/layout.py:14-38) for a 0/1 mask, both orientations.  One workgroup
+// of 16 wavefronts scans the mask twice (row-major, then column-major) with
+// wave ballots + popcounts; the row-major ordinal of every cell is parked in a
+// workspace so the column pass can attach it to its pairs.
+//
+// Schedule: see bsa.h.  A serial first-fit pass over the groups (one lane)
+// fixes each group's first slot, then all lanes fill the slots.
+#include "bsa_device.hpp"
+#include "bsa_internal.hpp"
+
+namespace bsa {
+
+constexpr int LB_THREADS = 1024;
+constexpr int LB_WAVES = LB_THREADS / WAVE;
+
+// Exclusive position of this thread's flag among the flags of the workgroup,
+// and the workgroup total.  `carry` is the running count of earlier tiles.
+__device__ __forceinline__ int tile_scan(bool flag, int *wave_tot, int &total)
+{
+    unsigned long long bal = __ballot(flag);
+    int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    int lane_prefix = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_tot[wave] = __popcll(bal);
+    __syncthreads();
+    int wave_prefix = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < LB_WAVES; ++w) {
+        int t = wave_tot[w];
+        wave_prefix += (w < wave) ? t : 0;
+        tot += t;
+    }
+    __syncthreads();
+    total = tot;
+    return wave_prefix + lane_prefix;
+}
+
+__global__ __launch_bounds__(LB_THREADS) void layout_build_kernel(
+    const uint8_t *__restrict__ mask, int R, int C,
+    int2 *__restrict__ row_blocks, int *__restrict__ row_off,
+    int2 *__restrict__ col_blocks, int *__restrict__ col_off,
+    int *__restrict__ nnz_out, int *__restrict__ ordinal_of)
+{
+    __shared__ int wave_tot[LB_WAVES];
+    const int n = R * C;
+    const int tid = (int)threadIdx.x;
+
+    // pass 1: row-major order -> row table, ordinals
+    int carry = 0;
+    for (int base = 0; base < n; base += LB_THREADS) {
+        int t = base + tid;
+        bool nz = t < n && mask[t] != 0;
+        int total;
+        int ord = carry + tile_scan(nz, wave_tot, total);
+        if (t < n) {
+            int r = t / C, c = t - r * C;
+            ordinal_of[t] = ord;
+            if (c == 0) row_off[r] = ord;
+            if (nz) row_blocks[ord] = make_int2(ord, (int)(((unsigned)r << 16) + (unsigned)c));
+        }
+        carry += total;
+    }
+    if (tid == 0) {
+        row_off[R] = carry;
+        col_off[C] = carry;
+        nnz_out[0] = carry;
+    }
+    __syncthreads();   // ordinal_of is re-read below by other lanes of this workgroup
+
+    // pass 2: column-major order -> column table
+    carry = 0;
+    for (int base = 0; base < n; base += LB_THREADS) {
+        int t = base + tid;
+        int c = t / R, r = t - c * R;
+        int cell = r * C + c;
+        bool nz = t < n && mask[cell] != 0;
+        int total;
+        int pos = carry + tile_scan(nz, wave_tot, total);
+        if (t < n) {
+            if (r == 0) col_off[c] = pos;
+            if (nz) col_blocks[pos] = make_int2(ordinal_of[cell], (int)(((unsigned)r << 16) + (unsigned)c));
+        }
+        carry += total;
+    }
+}
+
+// ---- schedule -------------------------------------------------------------
+
+__device__ __forceinline__ int waves_of_group(int len, int cap, int waves)
+{
+    int nw = (len + cap - 1) / cap;
+    nw = nw < 1 ? 1 : nw;
+    return nw > waves ? waves : nw;
+}
+
+__global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
+    const int *__restrict__ offsets, int groups, int cap, int waves,
+    int4 *__restrict__ sched, int capacity, int *__restrict__ n_wgs_out, int *__restrict__ first_slot)
+{
+    __shared__ int total_slots;
+    const int tid = (int)threadIdx.x;
+    // first-fit: a team never straddles a workgroup boundary
+    if (tid == 0) {
+        int pos = 0;
+        for (int g = 0; g < groups; ++g) {
+            int nw = waves_of_group(offsets[g + 1] - offsets[g], cap, waves);
+            int in_wg = pos % waves;
+            if (in_wg + nw > waves) pos += waves - in_wg;
+            first_slot[g] = pos;
+            pos += nw;
+        }
+        int n_wgs = (pos + waves - 1) / waves;
+        total_slots = n_wgs * waves;
+        n_wgs_out[0] = n_wgs;
+    }
+    __syncthreads();
+    const int slots = total_slots < capacity ? total_slots : capacity;
+    for (int s = tid; s < slots; s += LB_THREADS) sched[s] = make_int4(-1, 0, 0, 0);
+    __syncthreads();
+    for (int g = tid; g < groups; g += LB_THREADS) {
+        int lo = offsets[g], len = offsets[g + 1] - lo;
+        int nw = waves_of_group(len, cap, waves);
+        int s0 = first_slot[g];
+        for (int t = 0; t < nw; ++t) {
+            int b = lo + (int)(((long long)len * t) / nw);
+            int e = lo + (int)(((long long)len * (t + 1)) / nw);
+            if (s0 + t < capacity) sched[s0 + t] = make_int4(g, b, e, (s0 % waves) | (nw << 8));
+        }
+    }
+}
+
+// ---- launchers ------------------------------------------------------------
+
+hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_blocks,
+                               int32_t *row_off, int32_t *col_blocks, int32_t *col_off,
+                               int32_t *nnz_out, void *workspace, hipStream_t stream)
+{
+    layout_build_kernel<<<1, LB_THREADS, 0, stream>>>(mask, R, C, (int2 *)row_blocks, row_off,
+                                                     (int2 *)col_blocks, col_off, nnz_out,
+                                                     (int *)workspace);
+    return hipGetLastError();
+}
+
+hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
+                                 int32_t *sched, int64_t capacity, int32_t *n_wgs_out,
+                                 hipStream_t stream)
+{
+    // the tail of the buffer parks the first slot of every group
+    int64_t slot_capacity = capacity - (groups + 3) / 4;
+    int *first_slot = sched + 4 * slot_capacity;
+    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, (int4 *)sched,
+                                                       (int)slot_capacity, n_wgs_out, first_slot);
+    return hipGetLastError();
+}
+
+}  // namespace bsa

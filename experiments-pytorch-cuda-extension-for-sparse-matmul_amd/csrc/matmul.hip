@@ -1,0 +1,547 @@
+// SDD / DSD / DDS block-sparse matmul for gfx950.
+//
+// Replaces the three kernels of sparse/native/sparse_smm_gpu.cu:22-267 and the
+// unfinished fp16 twin sparse/native/sparse_hmm_gpu.cu:26-317.  Nothing of
+// their structure is kept: every nonzero 32x32 block is one MFMA tile owned by
+// ONE wavefront (v_mfma_f32_32x32x16_f16, fp32 accumulate; v_mfma_f32_32x32x2_f32
+// for fp32), operands whose contraction index is contiguous in memory go
+// straight from global memory into MFMA registers with 16-byte loads, operands
+// whose contraction index is the slow one pass through a wave-private LDS tile
+// and come back transposed with ds_read_b64_tr_b16.  No workgroup barrier sits
+// in any inner loop.
+//
+// Work distribution: a schedule (see bsa.h) hands every wavefront a chunk of
+// consecutive table pairs of one group.  SDD: the chunk's blocks share the
+// block row, whose dense rows are kept in registers.  DSD/DDS ("group walk"):
+// the waves of a team accumulate partial 32x64 tiles and reduce through LDS.
+//
+// MFMA roles.  Of the two operands the one indexed by the accumulator REGISTER
+// (v) is fed through perm16 so a lane ends up with 16 consecutive output
+// elements; it is always the operand that runs along the contiguous dimension
+// of the output.  The other operand is indexed by the lane.
+#include "bsa_device.hpp"
+#include "bsa_internal.hpp"
+#include "../../include/bsa.h"
+
+namespace bsa {
+
+constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles, reused for the fp32 partial tile
+constexpr int GW_DENSE_LD = 72;         // halves per row of the staged 32 x 64 dense tile
+constexpr int SDD_LDS_PER_WAVE = 4096;  // two 32 x 32 half tiles
+
+// ---------------------------------------------------------------------------
+// 32 x 32 fp16 operand tiles: 2 x 16 bytes per lane either way.
+// ---------------------------------------------------------------------------
+
+// contraction index contiguous: src -> element [index 0][k 0], row stride ld
+template <bool PERMUTED>
+__device__ __forceinline__ void ldg_tile_kc(const half_t *src, size_t ld, uint4 (&raw)[2])
+{
+    int l = lane_id();
+    int i = PERMUTED ? perm16(l & 31) : (l & 31);
+    const half_t *p = src + (size_t)i * ld + 8 * (l >> 5);
+    raw[0] = ldg16(p);
+    raw[1] = ldg16(p + 16);
+}
+
+// contraction index is the slow one: src -> element [k 0][index 0], row stride ld
+__device__ __forceinline__ void ldg_tile_ks(const half_t *src, size_t ld, uint4 (&raw)[2])
+{
+    int l = lane_id();
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        int c = l + 64 * q;
+        raw[q] = ldg16(src + (size_t)(c >> 2) * ld + 8 * (c & 3));
+    }
+}
+
+__device__ __forceinline__ void lds_put_tile32(half_t *tile, const uint4 (&raw)[2])
+{
+    int l = lane_id();
+    *reinterpret_cast<uint4 *>(tile + 8 * l) = raw[0];
+    *reinterpret_cast<uint4 *>(tile + 8 * (l + 64)) = raw[1];
+}
+
+// ---------------------------------------------------------------------------
+// SDD fp16
+// ---------------------------------------------------------------------------
+template <bool A_KC, bool B_KC, int KBT>
+__global__ __launch_bounds__(512) void sdd_f16_kernel(
+    const half_t *__restrict__ a, const half_t *__restrict__ b, half_t *__restrict__ c,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int nnz, int M, int N, int K)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    if (e.group < 0 || e.begin >= e.end) return;
+
+    half_t *tile_a = reinterpret_cast<half_t *>(lds_raw + (size_t)w * SDD_LDS_PER_WAVE);
+    half_t *tile_b = tile_a + BS2;
+    const half_t *ab = a + (size_t)batch * M * K;
+    const half_t *bb = b + (size_t)batch * N * K;
+    half_t *cb = c + (size_t)batch * nnz * BS2;
+    const int r = e.group;
+
+    auto load_a = [&](int kb, uint4(&raw)[2]) {
+        if (A_KC) ldg_tile_kc<false>(ab + (size_t)(BS * r) * K + BS * kb, K, raw);
+        else ldg_tile_ks(ab + (size_t)(BS * kb) * M + BS * r, M, raw);
+    };
+    auto load_b = [&](int cblk, int kb, uint4(&raw)[2]) {
+        if (B_KC) ldg_tile_kc<true>(bb + (size_t)(BS * cblk) * K + BS * kb, K, raw);
+        else ldg_tile_ks(bb + (size_t)(BS * kb) * N + BS * cblk, N, raw);
+    };
+    auto operands_a = [&](const uint4(&raw)[2], h8(&op)[2]) {
+        if (A_KC) { op[0] = as_h8(raw[0]); op[1] = as_h8(raw[1]); return; }
+        wave_lds_fence();
+        lds_put_tile32(tile_a, raw);
+        wave_lds_fence();
+        op[0] = lds_operand_tr<false>(tile_a, BS, 0, 0);
+        op[1] = lds_operand_tr<false>(tile_a, BS, 0, 1);
+    };
+    auto operands_b = [&](const uint4(&raw)[2], h8(&op)[2]) {
+        if (B_KC) { op[0] = as_h8(raw[0]); op[1] = as_h8(raw[1]); return; }
+        wave_lds_fence();
+        lds_put_tile32(tile_b, raw);
+        wave_lds_fence();
+        op[0] = lds_operand_tr<true>(tile_b, BS, 0, 0);
+        op[1] = lds_operand_tr<true>(tile_b, BS, 0, 1);
+    };
+    auto store = [&](int idx, const f16v &acc) {
+        uint4 lo, hi;
+        pack16(acc, lo, hi);
+        half_t *o = cb + (size_t)idx * BS2 + (l & 31) * BS + 16 * (l >> 5);
+        stg16(o, lo);
+        stg16(o + 8, hi);
+    };
+
+    if (KBT > 0) {
+        // dense rows of this block row stay in registers for the whole chunk
+        h8 aop[KBT > 0 ? KBT : 1][2];
+#pragma unroll
+        for (int kb = 0; kb < KBT; ++kb) {
+            uint4 raw[2];
+            load_a(kb, raw);
+            operands_a(raw, aop[kb]);
+        }
+        uint4 braw[2][KBT > 0 ? KBT : 1][2];
+        BlockDesc d[2];
+        d[0] = blocks[e.begin];
+#pragma unroll
+        for (int kb = 0; kb < KBT; ++kb) load_b(d[0].col(), kb, braw[0][kb]);
+        for (int p = e.begin; p < e.end; p += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                if (p + u < e.end) {
+                    if (p + u + 1 < e.end) {
+                        d[u ^ 1] = blocks[p + u + 1];
+#pragma unroll
+                        for (int kb = 0; kb < KBT; ++kb) load_b(d[u ^ 1].col(), kb, braw[u ^ 1][kb]);
+                    }
+                    f16v acc = {0};
+#pragma unroll
+                    for (int kb = 0; kb < KBT; ++kb) {
+                        h8 bop[2];
+                        operands_b(braw[u][kb], bop);
+                        acc = mfma_f16(bop[0], aop[kb][0], acc);
+                        acc = mfma_f16(bop[1], aop[kb][1], acc);
+                    }
+                    store(d[u].idx, acc);
+                }
+            }
+        }
+    } else {
+        const int kbs = K / BS;
+        for (int p = e.begin; p < e.end; ++p) {
+            const BlockDesc d = blocks[p];
+            f16v acc = {0};
+            uint4 araw[2], braw[2];
+            load_a(0, araw);
+            load_b(d.col(), 0, braw);
+            for (int kb = 0; kb < kbs; ++kb) {
+                h8 aop[2], bop[2];
+                operands_a(araw, aop);
+                operands_b(braw, bop);
+                if (kb + 1 < kbs) {
+                    load_a(kb + 1, araw);
+                    load_b(d.col(), kb + 1, braw);
+                }
+                acc = mfma_f16(bop[0], aop[0], acc);
+                acc = mfma_f16(bop[1], aop[1], acc);
+            }
+            store(d.idx, acc);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// fp32 operand tiles: 16 floats per lane, k = 16 * (lane / 32) + 0..15 of one
+// index.  Both memory orientations load straight into registers.
+// ---------------------------------------------------------------------------
+template <bool KC, bool PERMUTED>
+__device__ __forceinline__ void ldg_tile_f32(const float *src, size_t ld, float (&v)[16])
+{
+    int l = lane_id();
+    int i = PERMUTED ? perm16(l & 31) : (l & 31);
+    int k0 = 16 * (l >> 5);
+    if (KC) {   // src -> [index 0][k 0]
+        const float4 *p = reinterpret_cast<const float4 *>(src + (size_t)i * ld + k0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            float4 x = p[t];
+            v[4 * t] = x.x; v[4 * t + 1] = x.y; v[4 * t + 2] = x.z; v[4 * t + 3] = x.w;
+        }
+    } else {    // src -> [k 0][index 0]
+#pragma unroll
+        for (int t = 0; t < 16; ++t) v[t] = src[(size_t)(k0 + t) * ld + i];
+    }
+}
+
+__device__ __forceinline__ void store16_f32(float *o, const f16v &acc)
+{
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        *reinterpret_cast<float4 *>(o + 4 * t) =
+            make_float4(acc[4 * t], acc[4 * t + 1], acc[4 * t + 2], acc[4 * t + 3]);
+}
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(512) void sdd_f32_kernel(
+    const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ c,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int nnz, int M, int N, int K)
+{
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    if (e.group < 0 || e.begin >= e.end) return;
+    const float *ab = a + (size_t)batch * M * K;
+    const float *bb = b + (size_t)batch * N * K;
+    float *cb = c + (size_t)batch * nnz * BS2;
+    const int r = e.group, kbs = K / BS;
+
+    for (int p = e.begin; p < e.end; ++p) {
+        const BlockDesc d = blocks[p];
+        const int cblk = d.col();
+        f16v acc = {0};
+        for (int kb = 0; kb < kbs; ++kb) {
+            float av[16], bv[16];
+            if (A_KC) ldg_tile_f32<true, false>(ab + (size_t)(BS * r) * K + BS * kb, K, av);
+            else ldg_tile_f32<false, false>(ab + (size_t)(BS * kb) * M + BS * r, M, av);
+            if (B_KC) ldg_tile_f32<true, true>(bb + (size_t)(BS * cblk) * K + BS * kb, K, bv);
+            else ldg_tile_f32<false, true>(bb + (size_t)(BS * kb) * N + BS * cblk, N, bv);
+#pragma unroll
+            for (int t = 0; t < 16; ++t) acc = mfma_f32(bv[t], av[t], acc);
+        }
+        store16_f32(cb + (size_t)d.idx * BS2 + (l & 31) * BS + 16 * (l >> 5), acc);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Group walk (DSD and DDS).
+//
+//   out(x, y) = sum over the pairs of group g, sum over k of
+//               Sblk(x, k) * Dn(32 * kblk + k, y)
+//
+// x = 0..31 runs inside the group's block row/column of the sparse matrix,
+// y runs along the free dense dimension DN (a wave owns a strip of 64).
+//   S_KC  the stored block is [x][k] (row groups, kblk = pair column);
+//         otherwise [k][x] (column groups, kblk = pair row)
+//   D_KC  the dense operand is stored [DN][KT]; otherwise [KT][DN]
+//   DSD   output is [XT][DN] (y contiguous); otherwise (DDS) [DN][XT]
+// ---------------------------------------------------------------------------
+template <bool DSD>
+__device__ __forceinline__ size_t gw_out_offset(int g, int y0, int yt, int l, int DN, int XT)
+{
+    int h = l >> 5, i = l & 31;
+    if (DSD) return (size_t)(BS * g + i) * DN + y0 + 32 * yt + 16 * h;
+    return (size_t)(y0 + 32 * yt + i) * XT + BS * g + 16 * h;
+}
+
+// Team reduction through LDS + the leader's check.  Returns true for the wave
+// that has to store.  Every wave of the workgroup must call this once.
+__device__ __forceinline__ bool team_reduce(f16v (&acc)[2], const SchedEntry &e, int w,
+                                            unsigned char *lds_raw)
+{
+    const int l = lane_id();
+    const int slot0 = e.team & 0xFF, nw = e.team >> 8;
+    const bool active = e.group >= 0;
+    const bool leader = active && w == slot0;
+    float *mine = reinterpret_cast<float *>(lds_raw + (size_t)w * GW_LDS_PER_WAVE);
+    if (active && !leader) {
+        wave_lds_fence();
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) mine[(t * 16 + v) * WAVE + l] = acc[t][v];
+    }
+    __syncthreads();
+    if (leader) {
+        for (int o = 1; o < nw; ++o) {
+            const float *other = reinterpret_cast<const float *>(lds_raw + (size_t)(w + o) * GW_LDS_PER_WAVE);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[t][v] += other[(t * 16 + v) * WAVE + l];
+        }
+    }
+    return leader;
+}
+
+template <bool S_KC, bool D_KC, bool DSD, int DEPTH>
+__global__ __launch_bounds__(512) void gw_f16_kernel(
+    const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int nnz, int DN, int KT, int XT)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;   // whole workgroup leaves together
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const int y0 = 64 * (int)blockIdx.y;
+    const int ytiles = (DN - y0) >= 64 ? 2 : 1;
+
+    half_t *tile_s = reinterpret_cast<half_t *>(lds_raw + (size_t)w * GW_LDS_PER_WAVE);
+    half_t *tile_d = tile_s + BS2;
+    const half_t *spb = sp + (size_t)batch * nnz * BS2;
+    const half_t *dnb = dn + (size_t)batch * DN * KT;
+
+    // one pair's operands: 2 KB of the sparse block + up to 4 KB of the dense strip
+    struct Frag { uint4 s[2]; uint4 d0[2]; uint4 d1[2]; };
+
+    auto load = [&](int p, Frag &f) {
+        const BlockDesc d = blocks[p];
+        const int kblk = S_KC ? d.col() : d.row();
+        const half_t *sb = spb + (size_t)d.idx * BS2;
+        if (S_KC) ldg_tile_kc<!DSD>(sb, BS, f.s);
+        else ldg_tile_ks(sb, BS, f.s);
+        if (D_KC) {
+            const half_t *src = dnb + (size_t)y0 * KT + BS * kblk;
+            ldg_tile_kc<DSD>(src, KT, f.d0);
+            if (ytiles == 2) ldg_tile_kc<DSD>(src + (size_t)32 * KT, KT, f.d1);
+        } else {
+            const half_t *src = dnb + (size_t)(BS * kblk) * DN + y0;
+            const int chunks = 4 * ytiles;   // 16-byte chunks per k row
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                int cidx = l + 64 * q;
+                int row = cidx >> 3, ch = cidx & 7;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (ch < chunks) v = ldg16(src + (size_t)row * DN + 8 * ch);
+                (q < 2 ? f.d0[q & 1] : f.d1[q & 1]) = v;
+            }
+        }
+    };
+
+    f16v acc[2] = {{0}, {0}};
+
+    auto compute = [&](const Frag &f) {
+        h8 sop[2], dop[2][2];
+        if (!S_KC || !D_KC) {
+            wave_lds_fence();
+            if (!S_KC) lds_put_tile32(tile_s, f.s);
+            if (!D_KC) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    int cidx = l + 64 * q;
+                    *reinterpret_cast<uint4 *>(tile_d + (cidx >> 3) * GW_DENSE_LD + 8 * (cidx & 7)) =
+                        q < 2 ? f.d0[q & 1] : f.d1[q & 1];
+                }
+            }
+            wave_lds_fence();
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            sop[s] = S_KC ? as_h8(f.s[s]) : lds_operand_tr<!DSD>(tile_s, BS, 0, s);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                dop[t][s] = D_KC ? as_h8(t == 0 ? f.d0[s] : f.d1[s])
+                                 : lds_operand_tr<DSD>(tile_d, GW_DENSE_LD, 32 * t, s);
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if (DSD) {
+                acc[0] = mfma_f16(dop[0][s], sop[s], acc[0]);
+                if (ytiles == 2) acc[1] = mfma_f16(dop[1][s], sop[s], acc[1]);
+            } else {
+                acc[0] = mfma_f16(sop[s], dop[0][s], acc[0]);
+                if (ytiles == 2) acc[1] = mfma_f16(sop[s], dop[1][s], acc[1]);
+            }
+        }
+    };
+
+    if (e.group >= 0) {
+        Frag fr[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d)
+            if (e.begin + d < e.end) load(e.begin + d, fr[d]);
+        for (int p = e.begin; p < e.end; p += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                if (p + d < e.end) {
+                    compute(fr[d]);
+                    if (p + d + DEPTH < e.end) load(p + d + DEPTH, fr[d]);
+                }
+            }
+        }
+    }
+
+    if (team_reduce(acc, e, w, lds_raw)) {
+        half_t *ob = out + (size_t)batch * XT * DN;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (t < ytiles) {
+                uint4 lo, hi;
+                pack16(acc[t], lo, hi);
+                half_t *o = ob + gw_out_offset<DSD>(e.group, y0, t, l, DN, XT);
+                stg16(o, lo);
+                stg16(o + 8, hi);
+            }
+        }
+    }
+}
+
+template <bool S_KC, bool D_KC, bool DSD>
+__global__ __launch_bounds__(512) void gw_f32_kernel(
+    const float *__restrict__ sp, const float *__restrict__ dn, float *__restrict__ out,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int nnz, int DN, int KT, int XT)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const int y0 = 64 * (int)blockIdx.y;
+    const int ytiles = (DN - y0) >= 64 ? 2 : 1;
+    const float *spb = sp + (size_t)batch * nnz * BS2;
+    const float *dnb = dn + (size_t)batch * DN * KT;
+
+    f16v acc[2] = {{0}, {0}};
+    if (e.group >= 0) {
+        for (int p = e.begin; p < e.end; ++p) {
+            const BlockDesc d = blocks[p];
+            const int kblk = S_KC ? d.col() : d.row();
+            float sv[16], dv[2][16];
+            ldg_tile_f32<S_KC, !DSD>(spb + (size_t)d.idx * BS2, BS, sv);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (t < ytiles) {
+                    if (D_KC) ldg_tile_f32<true, DSD>(dnb + (size_t)(y0 + 32 * t) * KT + BS * kblk, KT, dv[t]);
+                    else ldg_tile_f32<false, DSD>(dnb + (size_t)(BS * kblk) * DN + y0 + 32 * t, DN, dv[t]);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                if (DSD) {
+                    acc[0] = mfma_f32(dv[0][k], sv[k], acc[0]);
+                    if (ytiles == 2) acc[1] = mfma_f32(dv[1][k], sv[k], acc[1]);
+                } else {
+                    acc[0] = mfma_f32(sv[k], dv[0][k], acc[0]);
+                    if (ytiles == 2) acc[1] = mfma_f32(sv[k], dv[1][k], acc[1]);
+                }
+            }
+        }
+    }
+    if (team_reduce(acc, e, w, lds_raw)) {
+        float *ob = out + (size_t)batch * XT * DN;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+            if (t < ytiles) store16_f32(ob + gw_out_offset<DSD>(e.group, y0, t, l, DN, XT), acc[t]);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// launchers
+// ---------------------------------------------------------------------------
+static inline unsigned grid_x(int n_swg, int batches) { return 8u * (unsigned)n_swg * (unsigned)((batches + 7) / 8); }
+
+template <bool A_KC, bool B_KC>
+static hipError_t launch_sdd_f16(const MatmulArgs &p, hipStream_t st)
+{
+    dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
+    size_t lds = (A_KC && B_KC) ? 0 : (size_t)p.sched_waves * SDD_LDS_PER_WAVE;
+#define BSA_SDD_ARGS (const half_t *)p.a, (const half_t *)p.b, (half_t *)p.c, (const BlockDesc *)p.blocks, \
+                     (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K
+    switch (p.K / BS) {
+        case 1: sdd_f16_kernel<A_KC, B_KC, 1><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        case 2: sdd_f16_kernel<A_KC, B_KC, 2><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        case 3: sdd_f16_kernel<A_KC, B_KC, 3><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        case 4: sdd_f16_kernel<A_KC, B_KC, 4><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        default: sdd_f16_kernel<A_KC, B_KC, 0><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+    }
+#undef BSA_SDD_ARGS
+    return hipGetLastError();
+}
+
+template <bool A_KC, bool B_KC>
+static hipError_t launch_sdd_f32(const MatmulArgs &p, hipStream_t st)
+{
+    dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
+    sdd_f32_kernel<A_KC, B_KC><<<grid, block, 0, st>>>(
+        (const float *)p.a, (const float *)p.b, (float *)p.c, (const BlockDesc *)p.blocks,
+        (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K);
+    return hipGetLastError();
+}
+
+hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t st)
+{
+    // op(a) is M x K: stored [M][K] (contraction contiguous) unless tr_a.
+    // op(b) is K x N: stored [N][K] (contraction contiguous) only with tr_b.
+    const bool a_kc = !p.tr_a, b_kc = p.tr_b;
+    if (dtype == BSA_F16) {
+        if (a_kc) return b_kc ? launch_sdd_f16<true, true>(p, st) : launch_sdd_f16<true, false>(p, st);
+        return b_kc ? launch_sdd_f16<false, true>(p, st) : launch_sdd_f16<false, false>(p, st);
+    }
+    if (a_kc) return b_kc ? launch_sdd_f32<true, true>(p, st) : launch_sdd_f32<true, false>(p, st);
+    return b_kc ? launch_sdd_f32<false, true>(p, st) : launch_sdd_f32<false, false>(p, st);
+}
+
+template <bool S_KC, bool D_KC, bool DSD>
+static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const MatmulArgs &p,
+                              int DN, int KT, int XT, hipStream_t st)
+{
+    dim3 grid(grid_x(p.sched_wgs, p.batches), (unsigned)((DN + 63) / 64)), block(64 * p.sched_waves);
+    size_t lds = (size_t)p.sched_waves * GW_LDS_PER_WAVE;
+    if (dtype == BSA_F16)
+        gw_f16_kernel<S_KC, D_KC, DSD, 3><<<grid, block, lds, st>>>(
+            (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+    else
+        gw_f32_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(
+            (const float *)sp, (const float *)dn, (float *)p.c, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+    return hipGetLastError();
+}
+
+hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream_t st)
+{
+    if (dsd) {
+        // sparse = a; row groups (stored block is [x][k]) unless tr_a.
+        // dense = b, op(b) is K x N: stored [K][N] unless tr_b -> D_KC = tr_b.
+        const bool s_kc = !p.tr_a, d_kc = p.tr_b;
+        const int DN = p.N, KT = p.K, XT = p.M;
+        if (s_kc) return d_kc ? launch_gw_t<true, true, true>(dtype, p.a, p.b, p, DN, KT, XT, st)
+                              : launch_gw_t<true, false, true>(dtype, p.a, p.b, p, DN, KT, XT, st);
+        return d_kc ? launch_gw_t<false, true, true>(dtype, p.a, p.b, p, DN, KT, XT, st)
+                    : launch_gw_t<false, false, true>(dtype, p.a, p.b, p, DN, KT, XT, st);
+    }
+    // DDS: sparse = b; column groups (stored block is [k][x]) unless tr_b.
+    // dense = a, op(a) is M x K: stored [M][K] unless tr_a -> D_KC = !tr_a.
+    const bool s_kc = p.tr_b, d_kc = !p.tr_a;
+    const int DN = p.M, KT = p.K, XT = p.N;
+    if (s_kc) return d_kc ? launch_gw_t<true, true, false>(dtype, p.b, p.a, p, DN, KT, XT, st)
+                          : launch_gw_t<true, false, false>(dtype, p.b, p.a, p, DN, KT, XT, st);
+    return d_kc ? launch_gw_t<false, true, false>(dtype, p.b, p.a, p, DN, KT, XT, st)
+                : launch_gw_t<false, false, false>(dtype, p.b, p.a, p, DN, KT, XT, st);
+}
+
+}  // namespace bsa

@@ -1,0 +1,426 @@
+// Block-sparse row softmax, forward and backward, for gfx950.
+//
+// Replaces sparse_softmax_32x32_forward_kernel / _backward_kernel and their two
+// block-wide reductions (sparse_softmax.cu:14-205).  The reference runs a
+// 1024-thread workgroup per ELEMENT row and makes three passes over global
+// memory; here a team of wavefronts owns a BLOCK row (32 element rows), every
+// wave pulls whole 32x32 blocks with 16-byte loads (a block is one or two fully
+// coalesced 1 KB requests per wave), keeps its chunk in registers, and the
+// data is read once and written once.
+//
+// Lane map of a block: 16-byte chunk c = lane + 64 * q of the block belongs to
+// element row c / LPR, so the LPR = 4 (fp16) or 8 (fp32) lanes of one row are
+// neighbours and row reductions are DPP moves (quad_perm, row_half_mirror); only
+// the (max, sum) of a row crosses waves, through 512 bytes of LDS per wave.
+//
+// Additions over the reference: `scale` (folded with log2(e) into one constant
+// so the exponential is v_exp_f32 of one fused multiply-add) and the causal
+// mask (global column > global row counts as -inf; only blocks on or above the
+// diagonal are touched by it).  Chunks longer than the register capacity fall
+// back to a two-pass walk (online max/sum, then re-read).
+#include "bsa_device.hpp"
+#include "bsa_internal.hpp"
+#include "../../include/bsa.h"
+
+namespace bsa {
+
+constexpr int SM_MAX_WAVES = 8;
+
+template <typename T> struct Chunk;
+template <> struct Chunk<half_t> {
+    static constexpr int NQ = 2;    // 16-byte chunks per lane per block
+    static constexpr int EPC = 8;   // elements per chunk
+    static constexpr int LPR = 4;   // lanes per element row
+    static __device__ __forceinline__ void unpack(const uint4 &r, float (&v)[8])
+    {
+        h8 h = __builtin_bit_cast(h8, r);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (float)h[i];
+    }
+    static __device__ __forceinline__ uint4 pack(const float (&v)[8])
+    {
+        h8 h;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[i] = (half_t)v[i];
+        return __builtin_bit_cast(uint4, h);
+    }
+};
+template <> struct Chunk<float> {
+    static constexpr int NQ = 4;
+    static constexpr int EPC = 4;
+    static constexpr int LPR = 8;
+    static __device__ __forceinline__ void unpack(const uint4 &r, float (&v)[4])
+    {
+        v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y);
+        v[2] = __uint_as_float(r.z); v[3] = __uint_as_float(r.w);
+    }
+    static __device__ __forceinline__ uint4 pack(const float (&v)[4])
+    {
+        return make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]),
+                          __float_as_uint(v[2]), __float_as_uint(v[3]));
+    }
+};
+
+// value of the neighbour lane selected by a DPP control word
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
+}
+
+// all-reduce over the LPR neighbouring lanes that hold one element row
+template <int LPR, typename Op>
+__device__ __forceinline__ float row_allreduce(float x, Op op)
+{
+    x = op(x, dpp<0xB1>(x));    // quad_perm [1,0,3,2]
+    x = op(x, dpp<0x4E>(x));    // quad_perm [2,3,0,1]
+    if (LPR == 8) x = op(x, dpp<0x141>(x));   // row_half_mirror: lane i <- lane 7 - i
+    return x;
+}
+
+struct MaxOp { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+struct AddOp { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------
+template <typename T, int CB>
+__global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
+    const T *__restrict__ x, T *__restrict__ y, const BlockDesc *__restrict__ blocks,
+    const SchedEntry *__restrict__ sched, int n_swg, int batches, int nnz,
+    float scale2 /* scale * log2(e) */, int causal)
+{
+    typedef Chunk<T> C;
+    constexpr int NQ = C::NQ, EPC = C::EPC, LPR = C::LPR;
+    constexpr int ROWS_PER_Q = WAVE / LPR;
+    __shared__ float2 stats[SM_MAX_WAVES][BS];
+
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const bool active = e.group >= 0;
+    const int n = active ? e.end - e.begin : 0;
+    const T *xb = x + (size_t)batch * nnz * BS2;
+    T *yb = y + (size_t)batch * nnz * BS2;
+    const int col0 = EPC * (l % LPR);          // first column of this lane's chunk inside a block
+    const int row0 = l / LPR;                  // element row of chunk q is row0 + q * ROWS_PER_Q
+    const float NEG_INF = -__builtin_inff();
+
+    // scaled scores of one chunk, masked
+    auto scaled = [&](const uint4 &raw, int q, int bcol, float (&v)[EPC]) {
+        C::unpack(raw, v);
+#pragma unroll
+        for (int i = 0; i < EPC; ++i) v[i] *= scale2;
+        if (causal && bcol >= e.group) {
+            int limit = (bcol > e.group) ? -1 : row0 + q * ROWS_PER_Q;   // last visible column in the block
+#pragma unroll
+            for (int i = 0; i < EPC; ++i)
+                if (col0 + i > limit) v[i] = NEG_INF;
+        }
+    };
+
+    float m[NQ], s[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) { m[q] = NEG_INF; s[q] = 0.f; }
+
+    uint4 raw[CB][NQ];
+    int bidx[CB], bcol[CB];
+    const bool resident = n <= CB;
+
+    if (resident) {
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+            if (j < n) {
+                const BlockDesc d = blocks[e.begin + j];
+                bidx[j] = d.idx; bcol[j] = d.col();
+                const T *src = xb + (size_t)d.idx * BS2;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) raw[j][q] = ldg16(src + (l + WAVE * q) * EPC);
+            }
+        }
+        // pass 1 (registers): row max
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+            if (j < n) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    float v[EPC];
+                    scaled(raw[j][q], q, bcol[j], v);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) m[q] = fmaxf(m[q], v[i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) m[q] = row_allreduce<LPR>(m[q], MaxOp());
+        // pass 2 (registers): exponentials in place, row sum
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+            if (j < n) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    float v[EPC];
+                    scaled(raw[j][q], q, bcol[j], v);
+                    const float mm = (m[q] == NEG_INF) ? 0.f : m[q];
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) {
+                        v[i] = exp2_fast(v[i] - mm);
+                        s[q] += v[i];
+                    }
+                    raw[j][q] = C::pack(v);
+                }
+            }
+        }
+    } else if (active) {
+        // streaming pass 1: online max / sum
+        for (int p = e.begin; p < e.end; ++p) {
+            const BlockDesc d = blocks[p];
+            const T *src = xb + (size_t)d.idx * BS2;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                float v[EPC];
+                scaled(ldg16(src + (l + WAVE * q) * EPC), q, d.col(), v);
+                float bm = v[0];
+#pragma unroll
+                for (int i = 1; i < EPC; ++i) bm = fmaxf(bm, v[i]);
+                const float nm = fmaxf(m[q], bm);
+                const float mm = (nm == NEG_INF) ? 0.f : nm;
+                float acc = s[q] * exp2_fast(m[q] - mm);
+#pragma unroll
+                for (int i = 0; i < EPC; ++i) acc += exp2_fast(v[i] - mm);
+                s[q] = acc;
+                m[q] = nm;
+            }
+        }
+        // lanes of a row hold different (m, s): bring them to the row max
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const float rm = row_allreduce<LPR>(m[q], MaxOp());
+            const float mm = (rm == NEG_INF) ? 0.f : rm;
+            s[q] *= exp2_fast(m[q] - mm);
+            m[q] = rm;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) s[q] = row_allreduce<LPR>(s[q], AddOp());
+
+    // team exchange of (max, sum) per element row
+    const int slot0 = e.team & 0xFF, nw = e.team >> 8;
+    if (active && (l % LPR) == 0) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) stats[w][row0 + q * ROWS_PER_Q] = make_float2(m[q], s[q]);
+    }
+    __syncthreads();
+    if (!active) return;
+
+    float f[NQ], gm[NQ], inv_s[NQ];   // factor for this wave's exponentials; row max; 1 / row sum
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+        float M = m[q], S = s[q];
+        if (nw > 1) {
+            M = NEG_INF;
+            for (int t = 0; t < nw; ++t) M = fmaxf(M, stats[slot0 + t][row0 + q * ROWS_PER_Q].x);
+            const float MM = (M == NEG_INF) ? 0.f : M;
+            S = 0.f;
+            for (int t = 0; t < nw; ++t) {
+                const float2 st = stats[slot0 + t][row0 + q * ROWS_PER_Q];
+                S += st.y * exp2_fast(st.x - MM);
+            }
+        }
+        const float MM = (M == NEG_INF) ? 0.f : M;
+        const float inv = S > 0.f ? 1.f / S : 0.f;
+        gm[q] = MM;
+        inv_s[q] = inv;
+        f[q] = exp2_fast(((m[q] == NEG_INF) ? 0.f : m[q]) - MM) * inv;
+        if (m[q] == NEG_INF) f[q] = 0.f;
+    }
+
+    if (resident) {
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+            if (j < n) {
+                T *dst = yb + (size_t)bidx[j] * BS2;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    float v[EPC];
+                    C::unpack(raw[j][q], v);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) v[i] *= f[q];
+                    stg16(dst + (l + WAVE * q) * EPC, C::pack(v));
+                }
+            }
+        }
+    } else {
+        // streaming pass 2: re-read, normalise, write
+        for (int p = e.begin; p < e.end; ++p) {
+            const BlockDesc d = blocks[p];
+            const T *src = xb + (size_t)d.idx * BS2;
+            T *dst = yb + (size_t)d.idx * BS2;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                float v[EPC];
+                scaled(ldg16(src + (l + WAVE * q) * EPC), q, d.col(), v);
+#pragma unroll
+                for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - gm[q]) * inv_s[q];
+                stg16(dst + (l + WAVE * q) * EPC, C::pack(v));
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward: dx = scale * (dy - sum_row(dy * y)) * y
+// ---------------------------------------------------------------------------
+template <typename T, int CB>
+__global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
+    const T *__restrict__ y, const T *__restrict__ dy, T *__restrict__ dx,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int nnz, float scale)
+{
+    typedef Chunk<T> C;
+    constexpr int NQ = C::NQ, EPC = C::EPC, LPR = C::LPR;
+    constexpr int ROWS_PER_Q = WAVE / LPR;
+    __shared__ float dots[SM_MAX_WAVES][BS];
+
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const bool active = e.group >= 0;
+    const int n = active ? e.end - e.begin : 0;
+    const size_t boff = (size_t)batch * nnz * BS2;
+    const int row0 = l / LPR;
+
+    float dot[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) dot[q] = 0.f;
+
+    uint4 ry[CB][NQ], rd[CB][NQ];
+    int bidx[CB];
+    const bool resident = n <= CB;
+    if (resident) {
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+            if (j < n) {
+                bidx[j] = blocks[e.begin + j].idx;
+                const size_t o = boff + (size_t)bidx[j] * BS2;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    ry[j][q] = ldg16(y + o + (l + WAVE * q) * EPC);
+                    rd[j][q] = ldg16(dy + o + (l + WAVE * q) * EPC);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+            if (j < n) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    float a[EPC], b[EPC];
+                    C::unpack(ry[j][q], a);
+                    C::unpack(rd[j][q], b);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
+                }
+            }
+        }
+    } else if (active) {
+        for (int p = e.begin; p < e.end; ++p) {
+            const size_t o = boff + (size_t)blocks[p].idx * BS2;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                float a[EPC], b[EPC];
+                C::unpack(ldg16(y + o + (l + WAVE * q) * EPC), a);
+                C::unpack(ldg16(dy + o + (l + WAVE * q) * EPC), b);
+#pragma unroll
+                for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
+
+    const int slot0 = e.team & 0xFF, nw = e.team >> 8;
+    if (active && (l % LPR) == 0) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) dots[w][row0 + q * ROWS_PER_Q] = dot[q];
+    }
+    __syncthreads();
+    if (!active) return;
+    if (nw > 1) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            float t = 0.f;
+            for (int o = 0; o < nw; ++o) t += dots[slot0 + o][row0 + q * ROWS_PER_Q];
+            dot[q] = t;
+        }
+    }
+
+    auto finish = [&](const uint4 &uy, const uint4 &ud, int q) {
+        float a[EPC], b[EPC];
+        C::unpack(uy, a);
+        C::unpack(ud, b);
+#pragma unroll
+        for (int i = 0; i < EPC; ++i) a[i] = scale * (b[i] - dot[q]) * a[i];
+        return C::pack(a);
+    };
+    if (resident) {
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+            if (j < n) {
+                const size_t o = boff + (size_t)bidx[j] * BS2;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) stg16(dx + o + (l + WAVE * q) * EPC, finish(ry[j][q], rd[j][q], q));
+            }
+        }
+    } else {
+        for (int p = e.begin; p < e.end; ++p) {
+            const size_t o = boff + (size_t)blocks[p].idx * BS2;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+                stg16(dx + o + (l + WAVE * q) * EPC,
+                      finish(ldg16(y + o + (l + WAVE * q) * EPC), ldg16(dy + o + (l + WAVE * q) * EPC), q));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// launchers
+// ---------------------------------------------------------------------------
+static inline unsigned grid_x(int n_swg, int batches) { return 8u * (unsigned)n_swg * (unsigned)((batches + 7) / 8); }
+
+hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t st)
+{
+    dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
+    const float scale2 = p.scale * 1.4426950408889634f;
+    if (dtype == BSA_F16)
+        softmax_fwd_kernel<half_t, 8><<<grid, block, 0, st>>>(
+            (const half_t *)p.x, (half_t *)p.out, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
+    else
+        softmax_fwd_kernel<float, 4><<<grid, block, 0, st>>>(
+            (const float *)p.x, (float *)p.out, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
+    return hipGetLastError();
+}
+
+hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t st)
+{
+    dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
+    if (dtype == BSA_F16)
+        softmax_bwd_kernel<half_t, 4><<<grid, block, 0, st>>>(
+            (const half_t *)p.x, (const half_t *)p.dy, (half_t *)p.out, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.scale);
+    else
+        softmax_bwd_kernel<float, 2><<<grid, block, 0, st>>>(
+            (const float *)p.x, (const float *)p.dy, (float *)p.out, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.scale);
+    return hipGetLastError();
+}
+
+}  // namespace bsa

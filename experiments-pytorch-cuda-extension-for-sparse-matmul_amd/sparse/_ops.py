@@ -1,0 +1,177 @@
+"""Host logic of the boundary: the Python twin of ``sparse_matmul`` in
+``sparse/native/sparse_kernels.cc:7-50`` (layout pick, M/N/K rules, batch
+flattening, output allocation, dtype dispatch) plus the argument checks the
+reference does not make.  ``sparse_matmul`` keeps the reference's positional
+signature (``native/sparse_ops.h:10-14``); the softmax entry points keep those of
+``sparse_softmax.cu:208-210,233-236`` with ``scale`` / ``causal`` appended.
+"""
+import torch
+
+from . import kernel as _k
+
+BLOCK = 32
+# tuning of the wavefront schedules: (target pairs per wavefront, wavefronts per workgroup)
+SCHEDULE_GROUP_WALK = (4, 8)
+SCHEDULE_SDD = (4, 4)
+SCHEDULE_SOFTMAX = (4, 8)
+
+_DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
+
+
+class Schedule:
+    """Device-resident wavefront schedule of one offset table."""
+
+    def __init__(self, offsets: torch.Tensor, nnz: int, cap: int, waves: int):
+        groups = offsets.numel() - 1
+        capacity = _k.lib.bsa_schedule_capacity(groups, nnz, cap, waves)
+        self.table = torch.empty(4 * capacity, dtype=torch.int32, device=offsets.device)
+        n_wgs = torch.empty(1, dtype=torch.int32, device=offsets.device)
+        with torch.cuda.device(offsets.device):
+            _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves,
+                                               self.table.data_ptr(), capacity, n_wgs.data_ptr(),
+                                               _k.current_stream()))
+        self.workgroups = int(n_wgs.item())
+        self.waves = waves
+        self.cap = cap
+
+
+def schedule_for(layout, kind):
+    """Schedule of a ``(blocks, offset_table)`` tuple, built on first use and kept
+    on the offset tensor (the reference's boundary passes only the two tensors)."""
+    blocks, offsets = layout
+    cache = getattr(offsets, "_bsa_schedules", None)
+    if cache is None:
+        cache = {}
+        offsets._bsa_schedules = cache
+    if kind not in cache:
+        cache[kind] = Schedule(offsets, blocks.numel() // 2, *kind)
+    return cache[kind]
+
+
+def _check_layout(layout, name):
+    blocks, offsets = layout
+    for t, what in ((blocks, "blocks"), (offsets, "offset_table")):
+        if not (isinstance(t, torch.Tensor) and t.dtype == torch.int32 and t.is_cuda and t.dim() == 1
+                and t.is_contiguous()):
+            raise ValueError(f"{name}.{what} must be a contiguous 1-D int32 tensor on the GPU")
+    if blocks.numel() % 2 or offsets.numel() < 2:
+        raise ValueError(f"{name} is malformed")
+
+
+def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=False):
+    """``c = op(a) @ op(b)`` with one of a, b, c block-sparse (sparse_kernels.cc:7-50)."""
+    if mode not in _k.MODES:
+        raise ValueError(f"mode must be one of 'sdd', 'dsd', 'dds', got {mode!r}")
+    if a.dtype != b.dtype or a.dtype not in _DTYPES:
+        raise TypeError(f"operands must both be float32 or both float16, got {a.dtype} and {b.dtype}")
+    if not (a.is_cuda and b.is_cuda) or a.device != b.device:
+        raise ValueError("operands must live on the same GPU")
+    _check_layout(row_layout, "row_layout")
+    _check_layout(col_layout, "col_layout")
+    trans_a, trans_b = bool(trans_a), bool(trans_b)
+
+    # sparse_kernels.cc:12 : which table the walk uses
+    use_row = mode == "sdd" or (mode == "dsd" and not trans_a) or (mode == "dds" and trans_b)
+    layout = row_layout if use_row else col_layout
+    if layout[0].device != a.device:
+        raise ValueError("layout tables and operands must live on the same GPU")
+    num_blocks = layout[0].numel() // 2
+    mask_rows, mask_cols = row_layout[1].numel() - 1, col_layout[1].numel() - 1
+    sparse_width = (layout[1].numel() - 1) * BLOCK                      # :14
+
+    a_dense, b_dense = mode[1] == "d", mode[2] == "d"
+    if a.dim() < (3 if a_dense else 4) or b.dim() < (3 if b_dense else 4):
+        raise ValueError("operands need at least one batch dimension "
+                         "(dense [..., rows, cols], sparse [..., nnz, 32, 32])")
+    for t, dense, name in ((a, a_dense, "a"), (b, b_dense, "b")):
+        if not dense and tuple(t.shape[-3:]) != (num_blocks, BLOCK, BLOCK):
+            raise ValueError(f"sparse operand {name} must be [..., {num_blocks}, 32, 32], got {tuple(t.shape)}")
+
+    # sparse_kernels.cc:17-19
+    size_m = a.size(-1 if trans_a else -2) if a_dense else sparse_width
+    size_n = b.size(-2 if trans_b else -1) if b_dense else sparse_width
+    size_k = b.size(-1 if trans_b else -2) if b_dense else a.size(-2 if trans_a else -1)
+    if a_dense and b_dense and a.size(-2 if trans_a else -1) != size_k:
+        raise ValueError("inner dimensions of op(a) and op(b) differ")
+
+    batch_a = tuple(a.shape[:-2] if a_dense else a.shape[:-3])
+    batch_b = tuple(b.shape[:-2] if b_dense else b.shape[:-3])
+    if batch_a != batch_b:
+        raise ValueError(f"batch dimensions differ: {batch_a} vs {batch_b} (no broadcasting)")
+    batches = 1
+    for s in batch_a:
+        batches *= s
+    if batches < 1:
+        raise ValueError("empty batch")
+
+    # :22-37 : flatten the batch, allocate the result
+    a = a.contiguous()
+    b = b.contiguous()
+    if mode[0] == "d":
+        shape = batch_a + (size_m, size_n)
+    else:
+        shape = batch_a + (num_blocks, BLOCK, BLOCK)
+    c = torch.empty(shape, dtype=a.dtype, device=a.device)
+
+    sched = schedule_for(layout, SCHEDULE_SDD if mode == "sdd" else SCHEDULE_GROUP_WALK)
+    with torch.cuda.device(a.device):
+        _k.check(_k.lib.bsa_matmul(
+            _k.MODES[mode], _DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), c.data_ptr(),
+            layout[0].data_ptr(), layout[1].data_ptr(), layout[1].numel() - 1,
+            sched.table.data_ptr(), sched.workgroups, sched.waves,
+            mask_rows, mask_cols, num_blocks, batches, size_m, size_n, size_k,
+            int(trans_a), int(trans_b), _k.current_stream()))
+    return c
+
+
+def _softmax_common(x, row_layout, col_layout, name):
+    if x.dtype not in _DTYPES:
+        raise TypeError(f"{name} must be float32 or float16, got {x.dtype}")
+    if not x.is_cuda:
+        raise ValueError(f"{name} must live on the GPU")
+    _check_layout(row_layout, "row_layout")
+    num_blocks = row_layout[0].numel() // 2
+    if x.dim() < 4 or tuple(x.shape[-3:]) != (num_blocks, BLOCK, BLOCK):
+        raise ValueError(f"{name} must be [..., {num_blocks}, 32, 32] with at least one batch "
+                         f"dimension, got {tuple(x.shape)}")
+    mask_rows = row_layout[1].numel() - 1
+    mask_cols = col_layout[1].numel() - 1 if col_layout is not None else 65535
+    batches = x.numel() // max(num_blocks * BLOCK * BLOCK, 1) if num_blocks else 1
+    return num_blocks, mask_rows, mask_cols, max(batches, 1)
+
+
+def sparse_softmax_forward(x, row_blocks, row_table, scale=1.0, causal=False, col_layout=None):
+    """``y = softmax(scale * x)`` over the stored blocks of each row (sparse_softmax.cu:208-231)."""
+    row_layout = (row_blocks, row_table)
+    nnz, mask_rows, mask_cols, batches = _softmax_common(x, row_layout, col_layout, "x")
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    if nnz == 0 or x.numel() == 0:
+        return y
+    sched = schedule_for(row_layout, SCHEDULE_SOFTMAX)
+    with torch.cuda.device(x.device):
+        _k.check(_k.lib.bsa_softmax_forward(
+            _DTYPES[x.dtype], x.data_ptr(), y.data_ptr(), row_blocks.data_ptr(), row_table.data_ptr(),
+            sched.table.data_ptr(), sched.workgroups, sched.waves, mask_rows, mask_cols, nnz, batches,
+            float(scale), int(bool(causal)), _k.current_stream()))
+    return y
+
+
+def sparse_softmax_backward(y, dy, row_blocks, row_table, scale=1.0, col_layout=None):
+    """``dx = scale * (dy - sum(dy * y)) * y`` per row (sparse_softmax.cu:233-258)."""
+    row_layout = (row_blocks, row_table)
+    nnz, mask_rows, mask_cols, batches = _softmax_common(y, row_layout, col_layout, "y")
+    if dy.shape != y.shape or dy.dtype != y.dtype or dy.device != y.device:
+        raise ValueError("dy must match y in shape, dtype and device")
+    y = y.contiguous()
+    dy = dy.contiguous()
+    dx = torch.empty_like(y)
+    if nnz == 0 or y.numel() == 0:
+        return dx
+    sched = schedule_for(row_layout, SCHEDULE_SOFTMAX)
+    with torch.cuda.device(y.device):
+        _k.check(_k.lib.bsa_softmax_backward(
+            _DTYPES[y.dtype], y.data_ptr(), dy.data_ptr(), dx.data_ptr(), row_blocks.data_ptr(),
+            row_table.data_ptr(), sched.table.data_ptr(), sched.workgroups, sched.waves,
+            mask_rows, mask_cols, nnz, batches, float(scale), _k.current_stream()))
+    return dx

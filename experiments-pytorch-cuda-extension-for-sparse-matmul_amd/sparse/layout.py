@@ -1,0 +1,79 @@
+"""``SparseLayout``: block mask -> block-index tables, dense <-> block-stack.
+
+Same class, attributes and methods as ``sparse/layout.py:5-57`` of the
+reference.  What changed underneath: the two tables are built by one device
+kernel from the uploaded mask (``bsa_layout_build``) instead of CPU torch ops
+and four host-to-device copies; ``to_sparse`` / ``to_dense`` are single gathers
+instead of Python loops over the blocks; ``to_dense`` fills absent blocks with
+zeros (the reference leaves them uninitialised); a bool mask means the same as
+the 0/1 integer mask.
+"""
+from typing import Tuple
+
+import torch
+
+from . import kernel as _k
+
+BLOCK = 32
+
+
+class SparseLayout:
+    def __init__(self, pattern: torch.Tensor, device=None):
+        if pattern.dim() != 2:
+            raise ValueError("pattern must be a 2-D block mask")
+        rows, cols = pattern.shape
+        if not (1 <= rows <= 32767 and 1 <= cols <= 65535):
+            raise ValueError("pattern shape must be within [1, 32767] x [1, 65535]")
+        if device is None:
+            device = pattern.device if pattern.is_cuda else torch.device("cuda", torch.cuda.current_device())
+        self.pattern = pattern
+        self.device = torch.device(device)
+
+        mask = (pattern != 0).to(device=self.device, dtype=torch.uint8).contiguous()
+        cells = rows * cols
+        row_blocks = torch.empty(2 * cells, dtype=torch.int32, device=self.device)
+        col_blocks = torch.empty(2 * cells, dtype=torch.int32, device=self.device)
+        row_offsets = torch.empty(rows + 1, dtype=torch.int32, device=self.device)
+        col_offsets = torch.empty(cols + 1, dtype=torch.int32, device=self.device)
+        nnz_dev = torch.empty(1, dtype=torch.int32, device=self.device)
+        workspace = torch.empty(_k.lib.bsa_layout_workspace_bytes(rows, cols), dtype=torch.uint8,
+                                device=self.device)
+        with torch.cuda.device(self.device):
+            _k.check(_k.lib.bsa_layout_build(
+                mask.data_ptr(), rows, cols, row_blocks.data_ptr(), row_offsets.data_ptr(),
+                col_blocks.data_ptr(), col_offsets.data_ptr(), nnz_dev.data_ptr(),
+                workspace.data_ptr(), _k.current_stream()))
+        nnz = int(nnz_dev.item())
+        self.num_blocks = nnz
+        # exact-size tensors: the boundary derives nnz from blocks.size(0) / 2 (sparse_kernels.cc:13)
+        self.row_layout: Tuple[torch.Tensor, torch.Tensor] = (row_blocks[:2 * nnz].clone(), row_offsets)
+        self.col_layout: Tuple[torch.Tensor, torch.Tensor] = (col_blocks[:2 * nnz].clone(), col_offsets)
+
+        packed = self.row_layout[0].view(-1, 2)[:, 1].long()
+        # [nnz, 2] (row, col) in row-major order == torch.nonzero(pattern) (layout.py:8)
+        self.sparse_positions = torch.stack((packed >> 16, packed & 0xFFFF), dim=1)
+        self._cell_index = (self.sparse_positions[:, 0] * cols + self.sparse_positions[:, 1])
+
+    def _index_on(self, device) -> torch.Tensor:
+        if self._cell_index.device != device:
+            return self._cell_index.to(device)
+        return self._cell_index
+
+    def to_sparse(self, x: torch.Tensor) -> torch.Tensor:
+        """``[..., R*32, C*32]`` -> ``[..., nnz, 32, 32]`` (layout.py:40-45)."""
+        rows, cols = self.pattern.shape
+        if tuple(x.shape[-2:]) != (rows * BLOCK, cols * BLOCK):
+            raise ValueError(f"expected [..., {rows * BLOCK}, {cols * BLOCK}], got {tuple(x.shape)}")
+        tiles = x.reshape(x.shape[:-2] + (rows, BLOCK, cols, BLOCK)).transpose(-3, -2)
+        tiles = tiles.reshape(x.shape[:-2] + (rows * cols, BLOCK, BLOCK))
+        return tiles.index_select(-3, self._index_on(x.device)).contiguous()
+
+    def to_dense(self, x: torch.Tensor) -> torch.Tensor:
+        """``[..., nnz, 32, 32]`` -> ``[..., R*32, C*32]``, absent blocks zero (layout.py:47-57)."""
+        rows, cols = self.pattern.shape
+        if tuple(x.shape[-3:]) != (self.num_blocks, BLOCK, BLOCK):
+            raise ValueError(f"expected [..., {self.num_blocks}, 32, 32], got {tuple(x.shape)}")
+        tiles = x.new_zeros(x.shape[:-3] + (rows * cols, BLOCK, BLOCK))
+        tiles.index_copy_(-3, self._index_on(x.device), x)
+        tiles = tiles.reshape(x.shape[:-3] + (rows, cols, BLOCK, BLOCK)).transpose(-3, -2)
+        return tiles.reshape(x.shape[:-3] + (rows * BLOCK, cols * BLOCK))

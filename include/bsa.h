@@ -1,0 +1,142 @@
+/*
+ * bsa.h - C ABI of libbsa_hip.so: block-sparse attention kernels for AMD
+ * Instinct MI355X (gfx950), 32x32 blocks.
+ *
+ * This library takes the place of the reference's torch C++ extension
+ * `sparse_ops` (pybind block sparse/native/sparse_kernels.cc:53-57, prototype
+ * native/sparse_ops.h:10-14).  Every entry point takes raw device pointers,
+ * plain sizes and a hipStream_t passed as void*; no torch types cross this
+ * boundary.  All functions
+ *   - return 0 on success and a negative BSA_ERR_* code otherwise,
+ *   - never synchronise, never allocate and never touch the null stream
+ *     unless the caller passes it,
+ *   - validate their arguments on the host before any launch; a message for
+ *     the last failure on the calling thread is kept for bsa_last_error().
+ *
+ * Table format (bit-exact with sparse/layout.py:21-36, decoded as in
+ * sparse/native/sparse_layout.cuh:13-21 but with a 16-bit column):
+ *   blocks   int32[2*nnz]  pairs (idx, (row << 16) + col); idx is the row-major
+ *                          ordinal of the block and addresses the block inside
+ *                          a sparse operand stored [batch, nnz, 32, 32]
+ *   offsets  int32[G+1]    first pair of every group: G = mask rows for the
+ *                          row layout, mask columns for the column layout
+ *
+ * Schedule format (new in this build): int32[4] per wavefront slot,
+ * (group, first pair, one-past-last pair, team), team = (slot of the team's
+ * first wave inside its workgroup) | (waves in the team << 8); group = -1
+ * marks an unused slot.  A workgroup owns `waves` consecutive slots; all waves
+ * that share a group sit in one workgroup so they can reduce through LDS.
+ */
+#ifndef BSA_H_
+#define BSA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BSA_BLOCK 32
+
+enum bsa_dtype { BSA_F32 = 0, BSA_F16 = 1 };
+enum bsa_mode { BSA_SDD = 0, BSA_DSD = 1, BSA_DDS = 2 };
+
+enum bsa_status {
+    BSA_OK = 0,
+    BSA_ERR_INVALID = -1,   /* argument validation failed; nothing was launched */
+    BSA_ERR_LAUNCH = -2,    /* the HIP runtime reported an error on launch      */
+    BSA_ERR_UNSUPPORTED = -3
+};
+
+/* Library version, major * 10000 + minor * 100 + patch. */
+int bsa_version(void);
+
+/* Message of the last failure on this thread ("" if none). Never NULL. */
+const char *bsa_last_error(void);
+
+/* ---- layout tables ------------------------------------------------------
+ * Device-side replacement of SparseLayout._create_layout (sparse/layout.py:14-38),
+ * both orientations in one launch.
+ *   mask         device uint8[R*C], row-major, nonzero = block present
+ *   row_blocks   device int32[2*R*C] (capacity; the first 2*nnz are written)
+ *   row_offsets  device int32[R+1]
+ *   col_blocks   device int32[2*R*C]
+ *   col_offsets  device int32[C+1]
+ *   nnz_out      device int32[1]
+ *   workspace    device, bsa_layout_workspace_bytes(R, C) bytes
+ * Limits: 1 <= R <= 32767, 1 <= C <= 65535 (the packed position is 16+16 bit
+ * in a signed int32).
+ */
+size_t bsa_layout_workspace_bytes(int mask_rows, int mask_cols);
+int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
+                     int32_t *row_blocks, int32_t *row_offsets,
+                     int32_t *col_blocks, int32_t *col_offsets,
+                     int32_t *nnz_out, void *workspace, void *stream);
+
+/* ---- wavefront schedule -------------------------------------------------
+ * Splits every group of a table into chunks of about `cap` pairs, one chunk
+ * per wavefront, and packs the wavefronts of a group into one workgroup of
+ * `waves` wavefronts (a group longer than cap*waves gets longer chunks).
+ * Empty groups get one wavefront with an empty chunk (it writes the zeros).
+ * No counterpart in the reference, whose grids are (nnz, B) and
+ * (B, M/32, N/32) (sparse/native/sparse_smm_gpu.cu:278-279).
+ *   sched        device int32[4 * bsa_schedule_capacity(...)]
+ *   n_wgs_out    device int32[1]: workgroups the schedule uses
+ */
+int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves);
+int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
+                       int32_t *sched, int64_t capacity, int32_t *n_wgs_out,
+                       void *stream);
+
+/* ---- block-sparse matmul -----------------------------------------------
+ * Replaces sparse_matmul's launch half: sparse_smm_32x32x32_kernel_wrapper and
+ * sparse_hmm_32x32x32_kernel_wrapper (sparse/native/sparse_kernels.h:10-24,
+ * sparse_smm_gpu.cu:270-293, sparse_hmm_gpu.cu:320-343).  The shape logic of
+ * sparse_kernels.cc:12-37 stays with the caller, which passes the result:
+ *   mode   BSA_SDD  c[b, idx]   = op(a)[b] (M x K) * op(b)[b] (K x N) on stored blocks
+ *          BSA_DSD  c[b] (MxN)  = op(S(a))[b] * op(b)[b]
+ *          BSA_DDS  c[b] (MxN)  = op(a)[b] * op(S(b))[b]
+ *   op(x) = x or its transpose (tr_a / tr_b); dense operands are contiguous
+ *   [batches, rows, cols] as stored, sparse ones [batches, nnz, 32, 32].
+ *   blocks/offsets/sched must be those of the layout the reference's rule
+ *   picks (sparse_kernels.cc:12): the ROW layout for sdd, for dsd without tr_a
+ *   and for dds with tr_b; the COLUMN layout otherwise.  `groups` is that
+ *   table's group count, `sched_wgs`/`sched_waves` describe its schedule.
+ *   M, N, K are the dims of op(a) (M x K) and op(b) (K x N); every dim that
+ *   runs along the sparse matrix must equal 32 * mask_rows / 32 * mask_cols
+ *   (after the transpose), the free dense dim must be a multiple of 32.
+ * fp16 accumulates in fp32.  Empty groups give zero rows / columns.
+ */
+int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
+               const int32_t *blocks, const int32_t *offsets, int groups,
+               const int32_t *sched, int sched_wgs, int sched_waves,
+               int mask_rows, int mask_cols, int nnz, int batches,
+               int M, int N, int K, int tr_a, int tr_b, void *stream);
+
+/* ---- block-sparse softmax ----------------------------------------------
+ * Replaces sparse_softmax_forward / sparse_softmax_backward
+ * (sparse_softmax.cu:208-258) and their kernels (:113-205), with two additions:
+ * the scores are multiplied by `scale` before the exponential, and with
+ * `causal` != 0 every element whose global column exceeds its global row
+ * counts as -inf.  x, y, dy, dx are [batches, nnz, 32, 32]; tables and schedule
+ * are those of the ROW layout.  Rows with nothing unmasked yield zeros.
+ *   forward : y  = softmax_row(scale * x)
+ *   backward: dx = scale * (dy - sum_row(dy * y)) * y
+ * Math is fp32 for both dtypes.
+ */
+int bsa_softmax_forward(int dtype, const void *x, void *y,
+                        const int32_t *row_blocks, const int32_t *row_offsets,
+                        const int32_t *sched, int sched_wgs, int sched_waves,
+                        int mask_rows, int mask_cols, int nnz, int batches,
+                        float scale, int causal, void *stream);
+int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
+                         const int32_t *row_blocks, const int32_t *row_offsets,
+                         const int32_t *sched, int sched_wgs, int sched_waves,
+                         int mask_rows, int mask_cols, int nnz, int batches,
+                         float scale, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BSA_H_ */

@@ -1,0 +1,105 @@
+"""GPU: the device table builder is bit-exact with the oracle; schedules are valid."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import layout_oracle as lo
+from helpers import mask_zoo
+
+pytestmark = pytest.mark.gpu
+
+
+def _layout(mask):
+    import sparse
+    return sparse.SparseLayout(torch.as_tensor(np.asarray(mask)))
+
+
+def _more_masks():
+    rng = np.random.RandomState(11)
+    out = list(mask_zoo())
+    out.append(("rand_256x256", (rng.rand(256, 256) < 0.1).astype(np.int64)))
+    out.append(("rand_100x37", (rng.rand(100, 37) < 0.5).astype(np.int64)))
+    out.append(("empty_33x65", np.zeros((33, 65), dtype=np.int64)))
+    out.append(("full_40x40", np.ones((40, 40), dtype=np.int64)))
+    wide = np.zeros((3, 300), dtype=np.int64)
+    wide[0, 256] = wide[1, 299] = wide[2, 0] = 1
+    out.append(("wide_3x300", wide))
+    return out
+
+
+@pytest.mark.parametrize("name,mask", _more_masks())
+def test_tables_bit_exact(name, mask):
+    mask = np.asarray(mask)
+    L = _layout(mask)
+    for tr, got in ((False, L.row_layout), (True, L.col_layout)):
+        blocks, offs = lo.create_layout(mask, tr)
+        assert got[0].dtype == torch.int32 and got[1].dtype == torch.int32 and got[0].is_cuda
+        assert np.array_equal(got[0].cpu().numpy(), blocks), (name, tr)
+        assert np.array_equal(got[1].cpu().numpy(), offs), (name, tr)
+    assert np.array_equal(L.sparse_positions.cpu().numpy(), lo.sparse_positions(mask))
+
+
+def test_bool_and_scaled_masks():
+    mask = np.array([[1, 0, 1], [0, 1, 0], [1, 1, 0]])
+    ref = lo.create_layout(mask)
+    for m in (torch.as_tensor(mask).bool(), torch.as_tensor(mask * 3), torch.as_tensor(mask).float()):
+        import sparse
+        L = sparse.SparseLayout(m)
+        assert np.array_equal(L.row_layout[0].cpu().numpy(), ref[0])
+        assert np.array_equal(L.row_layout[1].cpu().numpy(), ref[1])
+
+
+def test_golden_tables_on_device():
+    import workloads as wl
+    with open(os.path.join(os.path.dirname(__file__), "golden", "layout_tables.json")) as f:
+        golden = json.load(f)
+    masks = {"config1": wl.config1()["mask"], "config2": wl.mask_local_window(64, 2),
+             "config3_4": wl.mask_causal_local_strided(128), "config5": wl.mask_bigbird(256, wl._gen(5))}
+    for name, mask in masks.items():
+        L = _layout(mask.numpy())
+        g = golden[name]
+        assert L.num_blocks == g["nnz"]
+        for key, got in (("row", L.row_layout), ("col", L.col_layout)):
+            blocks = got[0].cpu().numpy().astype(np.int64)
+            w = np.arange(1, len(blocks) + 1, dtype=np.int64)
+            assert got[1].cpu().tolist() == g[key + "_offsets"]
+            assert int(blocks.sum()) == g[key + "_blocks_sum"]
+            assert int((blocks * w % 1000003).sum()) == g[key + "_blocks_wsum"]
+
+
+@pytest.mark.parametrize("name,mask", _more_masks())
+@pytest.mark.parametrize("cap,waves", [(4, 8), (1, 4), (16, 2), (3, 1)])
+def test_schedule_covers_every_pair_once(name, mask, cap, waves):
+    from sparse import _ops
+    mask = np.asarray(mask)
+    L = _layout(mask)
+    for layout in (L.row_layout, L.col_layout):
+        offs = layout[1].cpu().numpy()
+        groups = len(offs) - 1
+        s = _ops.Schedule(layout[1], layout[0].numel() // 2, cap, waves)
+        tab = s.table.cpu().numpy()[: 4 * s.workgroups * waves].reshape(-1, 4)
+        seen = np.zeros(max(int(offs[-1]), 1), dtype=np.int64)
+        group_seen = np.zeros(groups, dtype=np.int64)
+        for slot, (g, b, e, team) in enumerate(tab):
+            if g < 0:
+                continue
+            first, nw = team & 0xFF, team >> 8
+            wg, in_wg = divmod(slot, waves)
+            assert 0 <= g < groups and offs[g] <= b <= e <= offs[g + 1]
+            assert first <= in_wg < first + nw <= waves            # team sits inside one workgroup
+            leader = tab[wg * waves + first]
+            assert leader[0] == g                                   # same group as its leader
+            seen[b:e] += 1
+            if in_wg == first:
+                group_seen[g] += 1
+                # chunks of a team are consecutive and tile the group
+                chunks = tab[wg * waves + first: wg * waves + first + nw]
+                assert chunks[0][1] == offs[g] and chunks[-1][2] == offs[g + 1]
+                assert all(chunks[i][2] == chunks[i + 1][1] for i in range(nw - 1))
+                length = offs[g + 1] - offs[g]
+                assert nw == min(max(-(-length // cap), 1), waves)
+        assert np.all(seen[: int(offs[-1])] == 1)
+        assert np.all(group_seen == 1)                              # empty groups get a slot too
