@@ -1,0 +1,170 @@
+"""Benchmark of the block-sparse attention hot path on one MI355X.
+
+Workload (BASELINE.json's metric): fp16, seq 4096, block 32, 16 batch*heads, head
+dim 64, causal local-4 + every-8th-column mask (1530 of 16384 blocks, 9.3 %).
+A step is one pass of the three products over that batch:
+
+    SDD  scores = q @ k^T on the stored blocks       (reads q, k; writes 1530 blocks/head)
+    DSD  out    = probs @ v                           (reads 1530 blocks/head, v)
+    DDS  grad   = dy^T @ w  -> [16, 64, 4096]         (reads 1530 blocks/head, dy)
+
+`value` = nnz-block TFLOP/s = 3 * 2 * nnz * 32 * 32 * 64 * 16 flop / step time.
+The softmax (scale 1/8, causal) is timed in its own loop and reported in GB/s.
+Operands rotate over several resident sets so that the footprint exceeds the
+256 MB infinity cache and the figures are HBM figures.  Launches are replayed
+from HIP graphs (the Python call path costs more than a 10 us kernel).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sets S] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "experiments-pytorch-cuda-extension-for-sparse-matmul_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sets", type=int, default=4, help="operand sets to rotate over")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; the path shards over batch*heads with no "
+                 "communication, so --gpus N > 1 is not implemented (see DESIGN.md).")
+
+    import torch
+    import sparse
+    import workloads as wl
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    B, D = 16, 64
+    sets = []
+    for s in range(args.sets):
+        wk = wl.seq4096(batch=B, head_dim=D, seed=1004 + s)
+        sets.append({k: (v.to(dev) if hasattr(v, "to") else v) for k, v in wk.items()})
+    cpu_workload = wl.seq4096(batch=B, head_dim=D, seed=1004)
+    layout = sparse.SparseLayout(sets[0]["mask"])
+    nnz = layout.num_blocks
+    es = 2
+
+    flops_one = 2.0 * nnz * 32 * 32 * D * B
+    seq = 4096
+    bytes_alg = {
+        "sdd": (seq * D + seq * D) * B * es + nnz * 1024 * B * es,
+        "dsd": nnz * 1024 * B * es + seq * D * B * es + seq * D * B * es,
+        "dds": seq * D * B * es + nnz * 1024 * B * es + D * seq * B * es,
+        "softmax": 2 * nnz * 1024 * B * es,
+    }
+
+    ops = {
+        "sdd": lambda w: sparse.matmul(w["q"], w["k"], "sdd", layout, False, True),
+        "dsd": lambda w: sparse.matmul(w["scores"], w["v"], "dsd", layout, False, False),
+        "dds": lambda w: sparse.matmul(w["v"], w["w"], "dds", layout, True, False),
+        "softmax": lambda w: sparse.softmax(w["scores"], layout, 0.125, True),
+    }
+
+    def step(w):
+        return ops["sdd"](w), ops["dsd"](w), ops["dds"](w)
+
+    # parity spot check before timing: a fast wrong kernel is not a result
+    with torch.no_grad():
+        w0 = sets[0]
+        o = ops["dsd"](w0)
+        ref = torch.matmul(layout.to_dense(w0["scores"][:2]).float(), w0["v"][:2].float())
+        err = ((o[:2].float() - ref).abs().max() / ref.abs().max()).item()
+        assert err <= 2e-3, f"DSD parity check failed: {err}"
+
+    stream = torch.cuda.Stream()
+
+    def make_runner(fn, reps=1):
+        """One callable per operand set; each replays `reps` launches of fn on that set."""
+        runners = []
+        for w in sets:
+            if args.no_graph:
+                runners.append(lambda w=w: [fn(w) for _ in range(reps)])
+                continue
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(stream), torch.no_grad():
+                fn(w)                      # warm the caches / schedules outside capture
+                stream.synchronize()
+                with torch.cuda.graph(g, stream=stream):
+                    keep = [fn(w) for _ in range(reps)]
+            runners.append(lambda g=g, keep=keep: g.replay())
+        return runners
+
+    def timed(runners, n, warmup):
+        with torch.cuda.stream(stream), torch.no_grad():
+            for i in range(warmup):
+                runners[i % len(runners)]()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for i in range(n):
+                runners[i % len(runners)]()
+            e1.record(stream)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n    # ms per call
+
+    # headline: K steps of the three products
+    step_ms = timed(make_runner(step), args.steps, args.warmup)
+    value = 3 * flops_one / (step_ms * 1e-3) / 1e12
+
+    # per-kernel average launch duration: REPS launches per graph, events around the replays
+    REPS = 10
+    per_op = {}
+    for name, fn in ops.items():
+        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+        gbs = bytes_alg[name] / (ms * 1e-3) / 1e9
+        per_op[name] = {"us": round(ms * 1e3, 3), "GBps": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+                        "algorithmic_MB": round(bytes_alg[name] / 1e6, 3)}
+        if name != "softmax":
+            tf = flops_one / (ms * 1e-3) / 1e12
+            per_op[name]["nnz_TFLOPs"] = round(tf, 2)
+            per_op[name]["mfma_frac"] = round(tf / MFMA_F16_PEAK_TFLOPS, 4)
+
+    dominant = max(("sdd", "dsd", "dds"), key=lambda n: per_op[n]["us"])
+    roofline = {"kernel": dominant, "bound": "hbm", "achieved": per_op[dominant]["GBps"], "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": per_op[dominant]["hbm_frac"], "traffic": None}
+
+    result = {
+        "metric": "nnz-block TFLOP/s SDD/DSD/DDS fp16 @seq4096; softmax GB/s; % of roofline",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "seq4096_block32_causal-local4-stride8_nnz1530_bh16_d64: SDD(q,k^T)+DSD(p,v)+DDS(dy^T,w) per step",
+                   "operand_sets": args.sets, "launch": "eager" if args.no_graph else "hip-graph replay"},
+        "roofline": roofline,
+        "softmax": {"GBps": per_op["softmax"]["GBps"], "us": per_op["softmax"]["us"],
+                    "roofline": {"bound": "hbm", "achieved": per_op["softmax"]["GBps"], "peak": HBM_PEAK_GBS,
+                                 "unit": "GB/s", "frac": per_op["softmax"]["hbm_frac"], "traffic": None}},
+        "kernels": per_op,
+    }
+
+    if not args.no_cpu:
+        from oracle import cpu_baseline
+        heads = 2
+        cb = cpu_baseline.time_seq4096(cpu_workload, heads=heads, repeats=5)
+        cpu_tf = 3 * (flops_one / B * heads) / cb["matmul"] / 1e12
+        result["cpu_baseline"] = {
+            "value": round(cpu_tf, 5), "unit": "TFLOP/s", "cores": cb["cores"], "kind": "port",
+            "sample": f"{heads} of {B} heads of the same workload, masked-dense torch fp32 on the host, median of 5; "
+                      f"softmax on the same sample: {bytes_alg['softmax'] / B * heads / cb['softmax'] / 1e9:.3f} GB/s"}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

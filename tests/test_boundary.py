@@ -1,0 +1,89 @@
+"""CPU: the C-ABI library loads, exports what include/bsa.h declares, and validates on the host."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "bsa.h")
+
+
+@pytest.fixture(scope="module")
+def k():
+    import sparse.kernel as kernel
+    return kernel
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bsa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(k):
+    names = _declared()
+    assert names == sorted(k.SIGNATURES), "kernel.SIGNATURES must mirror include/bsa.h"
+    lib = ctypes.CDLL(k.LIBRARY_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert k.lib.bsa_version() >= 100
+    assert k.lib.bsa_last_error() is not None
+
+
+def test_missing_library_fails_loudly(k):
+    with pytest.raises(ImportError):
+        k.load_library("/nonexistent/libbsa_hip.so")
+
+
+def test_no_product_file_touches_the_oracle():
+    pkg = os.path.join(ROOT, "experiments-pytorch-cuda-extension-for-sparse-matmul_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h", ".cpp")):
+                assert "oracle" not in open(os.path.join(base, f)).read().lower(), f
+
+
+P = 0x1000  # any non-null address: validation fails before anything is dereferenced or launched
+
+
+def _matmul(k, mode=0, dtype=1, a=P, b=P, c=P, blocks=P, offs=P, groups=4, sched=P, wgs=1, waves=4,
+            R=4, C=4, nnz=5, batches=1, M=128, N=128, K=64, ta=0, tb=1):
+    return k.lib.bsa_matmul(mode, dtype, a, b, c, blocks, offs, groups, sched, wgs, waves, R, C, nnz,
+                            batches, M, N, K, ta, tb, None)
+
+
+@pytest.mark.parametrize("kw,needle", [
+    (dict(mode=7), "unknown mode"),
+    (dict(dtype=5), "unsupported dtype"),
+    (dict(a=None), "null pointer"),
+    (dict(sched=None), "schedule is null"),
+    (dict(K=48), "multiples of 32"),
+    (dict(M=96), "layout spans"),
+    (dict(groups=3), "groups"),
+    (dict(nnz=17), "does not fit"),
+    (dict(batches=0), "batches"),
+    (dict(waves=9), "waves per workgroup"),
+    (dict(wgs=0), "workgroups"),
+    (dict(mode=1, ta=0, tb=0, M=128, K=96, N=64), "op(sparse a)"),
+    (dict(mode=2, ta=0, tb=0, M=64, K=96, N=128), "op(sparse b)"),
+    (dict(R=0), "mask shape"),
+])
+def test_matmul_validation(k, kw, needle):
+    rc = _matmul(k, **kw)
+    assert rc < 0
+    assert needle in k.lib.bsa_last_error().decode()
+
+
+def test_other_entry_points_validate(k):
+    assert k.lib.bsa_layout_build(None, 4, 4, P, P, P, P, P, P, None) == -1
+    assert k.lib.bsa_layout_build(P, 40000, 4, P, P, P, P, P, P, None) == -1
+    assert "32767" in k.lib.bsa_last_error().decode()
+    assert k.lib.bsa_schedule_build(P, 4, 0, 4, P, 100, P, None) == -1
+    assert k.lib.bsa_schedule_build(P, 4, 4, 4, P, 3, P, None) == -1
+    assert "capacity" in k.lib.bsa_last_error().decode()
+    assert k.lib.bsa_softmax_forward(3, P, P, P, P, P, 1, 4, 4, 4, 5, 1, 1.0, 0, None) == -3
+    assert k.lib.bsa_softmax_forward(1, P, None, P, P, P, 1, 4, 4, 4, 5, 1, 1.0, 0, None) == -1
+    assert k.lib.bsa_softmax_backward(1, P, P, P, P, P, P, 1, 4, 4, 4, 5, 0, 1.0, None) == -1
+    assert k.lib.bsa_layout_workspace_bytes(4, 8) == 128
+    assert k.lib.bsa_schedule_capacity(4, 5, 4, 8) >= 2 * (4 + 1) + 8 + 1
