@@ -88,6 +88,12 @@ def main():
         err = ((o[:2].float() - ref).abs().max() / ref.abs().max()).item()
         assert err <= 2e-3, f"DSD parity check failed: {err}"
 
+    # plain copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters of a profiler run
+    cal_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    del cal_src, cal_dst
+
     stream = torch.cuda.Stream()
 
     def make_runner(fn, reps=1):

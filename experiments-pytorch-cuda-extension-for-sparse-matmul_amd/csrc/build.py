@@ -9,7 +9,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["api.hip", "layout_build.hip", "matmul.hip", "softmax.hip"]
-HEADERS = ["bsa_device.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
+HEADERS = ["bsa_device.hpp", "lds_tiles.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
 LIB = os.path.join(HERE, "libbsa_hip.so")
 
 FLAGS = [

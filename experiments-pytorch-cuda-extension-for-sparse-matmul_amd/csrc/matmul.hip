@@ -20,47 +20,17 @@
 // elements; it is always the operand that runs along the contiguous dimension
 // of the output.  The other operand is indexed by the lane.
 #include "bsa_device.hpp"
+#include "lds_tiles.hpp"
 #include "bsa_internal.hpp"
 #include "../../include/bsa.h"
 
 namespace bsa {
 
-constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles, reused for the fp32 partial tile
-constexpr int GW_DENSE_LD = 72;         // halves per row of the staged 32 x 64 dense tile
-constexpr int SDD_LDS_PER_WAVE = 4096;  // two 32 x 32 half tiles
-
-// ---------------------------------------------------------------------------
-// 32 x 32 fp16 operand tiles: 2 x 16 bytes per lane either way.
-// ---------------------------------------------------------------------------
-
-// contraction index contiguous: src -> element [index 0][k 0], row stride ld
-template <bool PERMUTED>
-__device__ __forceinline__ void ldg_tile_kc(const half_t *src, size_t ld, uint4 (&raw)[2])
-{
-    int l = lane_id();
-    int i = PERMUTED ? perm16(l & 31) : (l & 31);
-    const half_t *p = src + (size_t)i * ld + 8 * (l >> 5);
-    raw[0] = ldg16(p);
-    raw[1] = ldg16(p + 16);
-}
-
-// contraction index is the slow one: src -> element [k 0][index 0], row stride ld
-__device__ __forceinline__ void ldg_tile_ks(const half_t *src, size_t ld, uint4 (&raw)[2])
-{
-    int l = lane_id();
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        int c = l + 64 * q;
-        raw[q] = ldg16(src + (size_t)(c >> 2) * ld + 8 * (c & 3));
-    }
-}
-
-__device__ __forceinline__ void lds_put_tile32(half_t *tile, const uint4 (&raw)[2])
-{
-    int l = lane_id();
-    *reinterpret_cast<uint4 *>(tile + 8 * l) = raw[0];
-    *reinterpret_cast<uint4 *>(tile + 8 * (l + 64)) = raw[1];
-}
+constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + up to 5 KB), reused for the fp32 partial tile
+constexpr int GW_DENSE_LD = 80;         // halves per row of the staged [k][64] dense tile: 160-byte rows
+                                        // put 4 consecutive rows into 4 different 32-byte bank groups
+constexpr int SDD_KB_MAX = 4;           // k-blocks (of 32) whose operands stay resident per wave
+constexpr int SDD_LDS_PER_WAVE = 2048 * (1 + SDD_KB_MAX);   // a / result tile + one b tile per k-block
 
 // ---------------------------------------------------------------------------
 // SDD fp16
@@ -74,64 +44,63 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int batch, swg;
     if (!map_workgroup(n_swg, batches, batch, swg)) return;
-    const int w = wave_id(), l = lane_id();
+    const int w = wave_id();
     const int W = (int)(blockDim.x >> 6);
     const SchedEntry e = sched[swg * W + w];
     if (e.group < 0 || e.begin >= e.end) return;
 
     half_t *tile_a = reinterpret_cast<half_t *>(lds_raw + (size_t)w * SDD_LDS_PER_WAVE);
-    half_t *tile_b = tile_a + BS2;
+    half_t *tile_c = tile_a;            // the a tile is dead once its operands sit in registers
+    half_t *tile_b = tile_a + BS2;      // KBT (or 1) tiles
     const half_t *ab = a + (size_t)batch * M * K;
     const half_t *bb = b + (size_t)batch * N * K;
     half_t *cb = c + (size_t)batch * nnz * BS2;
     const int r = e.group;
 
+    // op(a) rows of the block row: [M][K] storage is contraction-contiguous, [K][M] is not
     auto load_a = [&](int kb, uint4(&raw)[2]) {
-        if (A_KC) ldg_tile_kc<false>(ab + (size_t)(BS * r) * K + BS * kb, K, raw);
-        else ldg_tile_ks(ab + (size_t)(BS * kb) * M + BS * r, M, raw);
+        if (A_KC) ldg_tile32(ab + (size_t)(BS * r) * K + BS * kb, K, raw);
+        else ldg_tile32(ab + (size_t)(BS * kb) * M + BS * r, M, raw);
     };
+    // op(b) columns of the block column: [N][K] storage is contraction-contiguous, [K][N] is not
     auto load_b = [&](int cblk, int kb, uint4(&raw)[2]) {
-        if (B_KC) ldg_tile_kc<true>(bb + (size_t)(BS * cblk) * K + BS * kb, K, raw);
-        else ldg_tile_ks(bb + (size_t)(BS * kb) * N + BS * cblk, N, raw);
+        if (B_KC) ldg_tile32(bb + (size_t)(BS * cblk) * K + BS * kb, K, raw);
+        else ldg_tile32(bb + (size_t)(BS * kb) * N + BS * cblk, N, raw);
     };
-    auto operands_a = [&](const uint4(&raw)[2], h8(&op)[2]) {
-        if (A_KC) { op[0] = as_h8(raw[0]); op[1] = as_h8(raw[1]); return; }
-        wave_lds_fence();
-        lds_put_tile32(tile_a, raw);
-        wave_lds_fence();
-        op[0] = lds_operand_tr<false>(tile_a, BS, 0, 0);
-        op[1] = lds_operand_tr<false>(tile_a, BS, 0, 1);
-    };
-    auto operands_b = [&](const uint4(&raw)[2], h8(&op)[2]) {
-        if (B_KC) { op[0] = as_h8(raw[0]); op[1] = as_h8(raw[1]); return; }
-        wave_lds_fence();
-        lds_put_tile32(tile_b, raw);
-        wave_lds_fence();
-        op[0] = lds_operand_tr<true>(tile_b, BS, 0, 0);
-        op[1] = lds_operand_tr<true>(tile_b, BS, 0, 1);
-    };
+    auto put_a = [&](half_t *t, const uint4(&raw)[2]) { if (A_KC) lds_put_kc<false>(t, raw); else lds_put_ks(t, raw); };
+    auto put_b = [&](half_t *t, const uint4(&raw)[2]) { if (B_KC) lds_put_kc<true>(t, raw); else lds_put_ks(t, raw); };
+    auto get_a = [&](const half_t *t, int s) { return A_KC ? lds_get_kc(t, s) : lds_get_ks<false>(t, s); };
+    auto get_b = [&](const half_t *t, int s) { return B_KC ? lds_get_kc(t, s) : lds_get_ks<true>(t, s); };
+    // the b operand feeds the accumulator-register index (through perm16), so a lane ends up
+    // with 16 consecutive columns of its row; the block leaves through LDS as whole 2 KB
     auto store = [&](int idx, const f16v &acc) {
-        uint4 lo, hi;
+        uint4 lo, hi, raw[2];
         pack16(acc, lo, hi);
-        half_t *o = cb + (size_t)idx * BS2 + (l & 31) * BS + 16 * (l >> 5);
-        stg16(o, lo);
-        stg16(o + 8, hi);
+        wave_lds_fence();
+        lds_put_result(tile_c, lo, hi);
+        wave_lds_fence();
+        lds_get_linear(tile_c, raw);
+        stg_tile32(cb + (size_t)idx * BS2, raw);
     };
 
     if (KBT > 0) {
-        // dense rows of this block row stay in registers for the whole chunk
-        h8 aop[KBT > 0 ? KBT : 1][2];
+        constexpr int KB = KBT > 0 ? KBT : 1;
+        h8 aop[KB][2];
 #pragma unroll
-        for (int kb = 0; kb < KBT; ++kb) {
+        for (int kb = 0; kb < KB; ++kb) {
             uint4 raw[2];
             load_a(kb, raw);
-            operands_a(raw, aop[kb]);
+            wave_lds_fence();
+            put_a(tile_a, raw);
+            wave_lds_fence();
+            aop[kb][0] = get_a(tile_a, 0);
+            aop[kb][1] = get_a(tile_a, 1);
         }
-        uint4 braw[2][KBT > 0 ? KBT : 1][2];
+        uint4 braw[2][KB][2];
         BlockDesc d[2];
         d[0] = blocks[e.begin];
 #pragma unroll
-        for (int kb = 0; kb < KBT; ++kb) load_b(d[0].col(), kb, braw[0][kb]);
+        for (int kb = 0; kb < KB; ++kb) load_b(d[0].col(), kb, braw[0][kb]);
         for (int p = e.begin; p < e.end; p += 2) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
@@ -139,15 +108,17 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
                     if (p + u + 1 < e.end) {
                         d[u ^ 1] = blocks[p + u + 1];
 #pragma unroll
-                        for (int kb = 0; kb < KBT; ++kb) load_b(d[u ^ 1].col(), kb, braw[u ^ 1][kb]);
+                        for (int kb = 0; kb < KB; ++kb) load_b(d[u ^ 1].col(), kb, braw[u ^ 1][kb]);
                     }
+                    wave_lds_fence();
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb) put_b(tile_b + kb * BS2, braw[u][kb]);
+                    wave_lds_fence();
                     f16v acc = {0};
 #pragma unroll
-                    for (int kb = 0; kb < KBT; ++kb) {
-                        h8 bop[2];
-                        operands_b(braw[u][kb], bop);
-                        acc = mfma_f16(bop[0], aop[kb][0], acc);
-                        acc = mfma_f16(bop[1], aop[kb][1], acc);
+                    for (int kb = 0; kb < KB; ++kb) {
+                        acc = mfma_f16(get_b(tile_b + kb * BS2, 0), aop[kb][0], acc);
+                        acc = mfma_f16(get_b(tile_b + kb * BS2, 1), aop[kb][1], acc);
                     }
                     store(d[u].idx, acc);
                 }
@@ -162,15 +133,16 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
             load_a(0, araw);
             load_b(d.col(), 0, braw);
             for (int kb = 0; kb < kbs; ++kb) {
-                h8 aop[2], bop[2];
-                operands_a(araw, aop);
-                operands_b(braw, bop);
+                wave_lds_fence();
+                put_a(tile_a, araw);
+                put_b(tile_b, braw);
+                wave_lds_fence();
                 if (kb + 1 < kbs) {
                     load_a(kb + 1, araw);
                     load_b(d.col(), kb + 1, braw);
                 }
-                acc = mfma_f16(bop[0], aop[0], acc);
-                acc = mfma_f16(bop[1], aop[1], acc);
+                acc = mfma_f16(get_b(tile_b, 0), get_a(tile_a, 0), acc);
+                acc = mfma_f16(get_b(tile_b, 1), get_a(tile_a, 1), acc);
             }
             store(d.idx, acc);
         }
@@ -313,28 +285,27 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     const half_t *spb = sp + (size_t)batch * nnz * BS2;
     const half_t *dnb = dn + (size_t)batch * DN * KT;
 
-    // one pair's operands: 2 KB of the sparse block + up to 4 KB of the dense strip
+    // one pair's operands: 2 KB of the sparse block + up to 4 KB of the dense strip,
+    // every request fully coalesced
     struct Frag { uint4 s[2]; uint4 d0[2]; uint4 d1[2]; };
 
     auto load = [&](int p, Frag &f) {
         const BlockDesc d = blocks[p];
         const int kblk = S_KC ? d.col() : d.row();
-        const half_t *sb = spb + (size_t)d.idx * BS2;
-        if (S_KC) ldg_tile_kc<!DSD>(sb, BS, f.s);
-        else ldg_tile_ks(sb, BS, f.s);
-        if (D_KC) {
+        ldg_tile32(spb + (size_t)d.idx * BS2, BS, f.s);
+        if (D_KC) {          // stored [DN][KT]: two 32 x 32 tiles, rows KT apart
             const half_t *src = dnb + (size_t)y0 * KT + BS * kblk;
-            ldg_tile_kc<DSD>(src, KT, f.d0);
-            if (ytiles == 2) ldg_tile_kc<DSD>(src + (size_t)32 * KT, KT, f.d1);
-        } else {
+            ldg_tile32(src, KT, f.d0);
+            if (ytiles == 2) ldg_tile32(src + (size_t)32 * KT, KT, f.d1);
+        } else {             // stored [KT][DN]: 32 rows of 64 (or 32) halves
             const half_t *src = dnb + (size_t)(BS * kblk) * DN + y0;
-            const int chunks = 4 * ytiles;   // 16-byte chunks per k row
+            const int pieces = 4 * ytiles;   // 16-byte pieces per k row
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 int cidx = l + 64 * q;
                 int row = cidx >> 3, ch = cidx & 7;
                 uint4 v = make_uint4(0, 0, 0, 0);
-                if (ch < chunks) v = ldg16(src + (size_t)row * DN + 8 * ch);
+                if (ch < pieces) v = ldg16(src + (size_t)row * DN + 8 * ch);
                 (q < 2 ? f.d0[q & 1] : f.d1[q & 1]) = v;
             }
         }
@@ -342,37 +313,34 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
 
     f16v acc[2] = {{0}, {0}};
 
+    // DSD: the dense strip feeds the accumulator-register index (perm16), the block the lane index;
+    // DDS: the other way round.
     auto compute = [&](const Frag &f) {
-        h8 sop[2], dop[2][2];
-        if (!S_KC || !D_KC) {
-            wave_lds_fence();
-            if (!S_KC) lds_put_tile32(tile_s, f.s);
-            if (!D_KC) {
+        wave_lds_fence();
+        if (S_KC) lds_put_kc<!DSD>(tile_s, f.s);
+        else lds_put_ks(tile_s, f.s);
+        if (D_KC) {
+            lds_put_kc<DSD>(tile_d, f.d0);
+            if (ytiles == 2) lds_put_kc<DSD>(tile_d + BS2, f.d1);
+        } else {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    int cidx = l + 64 * q;
-                    *reinterpret_cast<uint4 *>(tile_d + (cidx >> 3) * GW_DENSE_LD + 8 * (cidx & 7)) =
-                        q < 2 ? f.d0[q & 1] : f.d1[q & 1];
-                }
+            for (int q = 0; q < 4; ++q) {
+                int cidx = l + 64 * q;
+                *reinterpret_cast<uint4 *>(tile_d + (cidx >> 3) * GW_DENSE_LD + 8 * (cidx & 7)) =
+                    q < 2 ? f.d0[q & 1] : f.d1[q & 1];
             }
-            wave_lds_fence();
         }
+        wave_lds_fence();
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            sop[s] = S_KC ? as_h8(f.s[s]) : lds_operand_tr<!DSD>(tile_s, BS, 0, s);
+            const h8 sop = S_KC ? lds_get_kc(tile_s, s) : lds_get_ks<!DSD>(tile_s, s);
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-                dop[t][s] = D_KC ? as_h8(t == 0 ? f.d0[s] : f.d1[s])
-                                 : lds_operand_tr<DSD>(tile_d, GW_DENSE_LD, 32 * t, s);
-        }
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            if (DSD) {
-                acc[0] = mfma_f16(dop[0][s], sop[s], acc[0]);
-                if (ytiles == 2) acc[1] = mfma_f16(dop[1][s], sop[s], acc[1]);
-            } else {
-                acc[0] = mfma_f16(sop[s], dop[0][s], acc[0]);
-                if (ytiles == 2) acc[1] = mfma_f16(sop[s], dop[1][s], acc[1]);
+            for (int t = 0; t < 2; ++t) {
+                if (t < ytiles) {
+                    const h8 dop = D_KC ? lds_get_kc(tile_d + t * BS2, s)
+                                        : lds_operand_tr<DSD>(tile_d, GW_DENSE_LD, 32 * t, s);
+                    acc[t] = DSD ? mfma_f16(dop, sop, acc[t]) : mfma_f16(sop, dop, acc[t]);
+                }
             }
         }
     };
@@ -468,7 +436,7 @@ template <bool A_KC, bool B_KC>
 static hipError_t launch_sdd_f16(const MatmulArgs &p, hipStream_t st)
 {
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
-    size_t lds = (A_KC && B_KC) ? 0 : (size_t)p.sched_waves * SDD_LDS_PER_WAVE;
+    size_t lds = (size_t)p.sched_waves * SDD_LDS_PER_WAVE;
 #define BSA_SDD_ARGS (const half_t *)p.a, (const half_t *)p.b, (half_t *)p.c, (const BlockDesc *)p.blocks, \
                      (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K
     switch (p.K / BS) {
