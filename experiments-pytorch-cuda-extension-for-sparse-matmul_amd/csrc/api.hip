@@ -77,29 +77,40 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
 int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves)
 {
     if (groups < 1 || nnz < 0 || cap < 1 || waves < 1) return 0;
-    int64_t slots = 2 * ((int64_t)groups + nnz / cap + 1) + waves;
-    return slots + (groups + 3) / 4;
+    // waves: sum over parts of (len / cap + 1) <= nnz / cap + parts, parts <= nnz / (cap * waves) + groups;
+    // first-fit padding wastes less than the waves it pads for
+    int64_t slots = 2 * (2 * ((int64_t)nnz / cap) + groups + 1) + waves;
+    return slots + groups;   // one record per group in front
 }
 
-int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                       int32_t *sched, int64_t capacity, int32_t *n_wgs_out, void *stream)
+int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves, int allow_split,
+                       int32_t *sched, int64_t capacity, int32_t *counts_out, void *stream)
 {
-    if (!offsets || !sched || !n_wgs_out) return fail(BSA_ERR_INVALID, "bsa_schedule_build: null pointer argument");
+    if (!offsets || !sched || !counts_out) return fail(BSA_ERR_INVALID, "bsa_schedule_build: null pointer argument");
     if (groups < 1 || groups > 65535) return fail(BSA_ERR_INVALID, "bsa_schedule_build: %d groups outside [1, 65535]", groups);
     if (cap < 1) return fail(BSA_ERR_INVALID, "bsa_schedule_build: cap %d < 1", cap);
     if (waves < 1 || waves > MAX_WAVES)
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: waves %d outside [1, %d]", waves, MAX_WAVES);
-    if (capacity < 2 * ((int64_t)groups + 1) + waves + (groups + 3) / 4 || capacity > (1LL << 28))
+    if (capacity < 2 * ((int64_t)groups + 1) + waves + groups || capacity > (1LL << 28))
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: capacity %lld too small for %d groups (use bsa_schedule_capacity)",
                     (long long)capacity, groups);
-    return check_launch(bsa::launch_schedule_build(offsets, groups, cap, waves, sched, capacity, n_wgs_out,
-                                                   (hipStream_t)stream),
+    return check_launch(bsa::launch_schedule_build(offsets, groups, cap, waves, allow_split != 0, sched, capacity,
+                                                   counts_out, (hipStream_t)stream),
                         "bsa_schedule_build");
+}
+
+size_t bsa_matmul_workspace_bytes(int mode, int sched_tile_slots, int sched_split_groups,
+                                  int batches, int M, int N)
+{
+    if (mode == BSA_SDD || sched_tile_slots <= 0 || sched_split_groups <= 0 || batches < 1) return 0;
+    return bsa::gw_workspace_bytes(sched_tile_slots, sched_split_groups, batches, mode == BSA_DSD ? N : M);
 }
 
 int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
                const int32_t *blocks, const int32_t *offsets, int groups,
                const int32_t *sched, int sched_wgs, int sched_waves,
+               int sched_tile_slots, int sched_split_groups,
+               void *workspace, size_t workspace_bytes,
                int mask_rows, int mask_cols, int nnz, int batches,
                int M, int N, int K, int tr_a, int tr_b, void *stream)
 {
@@ -146,7 +157,15 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
     if ((free_dim + 63) / 64 > 65535)
         return fail(BSA_ERR_INVALID, "bsa_matmul: dense dimension %d is too large", free_dim);
 
-    bsa::MatmulArgs p{a, b, c, blocks, sched, sched_wgs, sched_waves, nnz, batches, M, N, K, tr_a != 0, tr_b != 0};
+    if (sched_tile_slots < 0 || sched_split_groups < 0 || (sched_tile_slots > 0) != (sched_split_groups > 0))
+        return fail(BSA_ERR_INVALID, "bsa_matmul: schedule split counts %d, %d are inconsistent",
+                    sched_tile_slots, sched_split_groups);
+    const size_t ws_need = bsa_matmul_workspace_bytes(mode, sched_tile_slots, sched_split_groups, batches, M, N);
+    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need))
+        return fail(BSA_ERR_INVALID, "bsa_matmul: workspace of %zu bytes needed, %zu given", ws_need, workspace_bytes);
+
+    bsa::MatmulArgs p{a, b, c, blocks, sched, groups, sched_wgs, sched_waves, sched_tile_slots, sched_split_groups,
+                      workspace, nnz, batches, M, N, K, tr_a != 0, tr_b != 0};
     if (nnz == 0 && mode == BSA_SDD) return BSA_OK;   // nothing to write
     hipError_t err = mode == BSA_SDD ? bsa::launch_sdd(dtype, p, (hipStream_t)stream)
                                      : bsa::launch_group_walk(dtype, mode == BSA_DSD, p, (hipStream_t)stream);
@@ -178,7 +197,7 @@ int bsa_softmax_forward(int dtype, const void *x, void *y,
                            sched_waves, mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
     if (nnz == 0) return BSA_OK;
-    bsa::SoftmaxArgs p{x, nullptr, y, row_blocks, sched, sched_wgs, sched_waves, nnz, batches, scale, causal != 0};
+    bsa::SoftmaxArgs p{x, nullptr, y, row_blocks, sched, mask_rows, sched_wgs, sched_waves, nnz, batches, scale, causal != 0};
     return check_launch(bsa::launch_softmax_forward(dtype, p, (hipStream_t)stream), "bsa_softmax_forward");
 }
 
@@ -192,7 +211,7 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
                            sched_waves, mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
     if (nnz == 0) return BSA_OK;
-    bsa::SoftmaxArgs p{y, dy, dx, row_blocks, sched, sched_wgs, sched_waves, nnz, batches, scale, false};
+    bsa::SoftmaxArgs p{y, dy, dx, row_blocks, sched, mask_rows, sched_wgs, sched_waves, nnz, batches, scale, false};
     return check_launch(bsa::launch_softmax_backward(dtype, p, (hipStream_t)stream), "bsa_softmax_backward");
 }
 

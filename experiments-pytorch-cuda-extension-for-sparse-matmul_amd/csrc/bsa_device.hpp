@@ -30,12 +30,31 @@ struct BlockDesc {
     __device__ __forceinline__ int col() const { return pos & 0xFFFF; }
 };
 
-// One wavefront slot of a schedule.
+// One wavefront slot of a schedule.  A group is cut into `parts` pieces, one team of
+// wavefronts each; a team sits inside one workgroup.
 struct SchedEntry {
     int group;   // -1: unused slot
     int begin;   // first pair of the chunk
     int end;     // one past the last pair
-    int team;    // (slot of the team's first wave in the workgroup) | (team waves << 8)
+    int team;    // see sched_team_word
+    __device__ __forceinline__ int first_wave() const { return team & 0xF; }           // slot of the team's first wave
+    __device__ __forceinline__ int team_waves() const { return (team >> 4) & 0xF; }
+    __device__ __forceinline__ int part() const { return (team >> 8) & 0xFFF; }
+    __device__ __forceinline__ int parts() const { return (int)((unsigned)team >> 20); }
+};
+
+constexpr int SCHED_MAX_PARTS = 4095;
+__host__ __device__ __forceinline__ int sched_team_word(int first_wave, int team_waves, int part, int parts)
+{
+    return first_wave | (team_waves << 4) | (part << 8) | (int)((unsigned)parts << 20);
+}
+
+// Per-group record in front of the slots.
+struct SchedGroup {
+    int first_slot;    // slot of part 0's first wave
+    int tile_slot;     // first partial-tile slot of a split group, else -1
+    int split_index;   // ordinal among the split groups, else -1
+    int parts;
 };
 
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63u); }

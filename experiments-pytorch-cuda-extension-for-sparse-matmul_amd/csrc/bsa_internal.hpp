@@ -11,21 +11,26 @@ hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_b
                                int32_t *nnz_out, void *workspace, hipStream_t stream);
 
 hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                                 int32_t *sched, int64_t capacity, int32_t *n_wgs_out,
-                                 hipStream_t stream);
+                                 int allow_split, int32_t *sched, int64_t capacity,
+                                 int32_t *counts_out, hipStream_t stream);
 
 struct MatmulArgs {
     const void *a, *b;
     void *c;
     const int32_t *blocks;
-    const int32_t *sched;
+    const int32_t *sched;      // group records, then wavefront slots
+    int groups;
     int sched_wgs, sched_waves;
+    int tile_slots, split_groups;   // partial tiles / counters one (batch, strip) needs
+    void *workspace;
     int nnz, batches;
     int M, N, K;
     bool tr_a, tr_b;
 };
 
 hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t stream);
+size_t gw_counter_bytes(int split_groups, int batches, int free_dim);
+size_t gw_workspace_bytes(int tile_slots, int split_groups, int batches, int free_dim);
 // group walk shared by DSD (dsd = true) and DDS
 hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream_t stream);
 
@@ -35,6 +40,7 @@ struct SoftmaxArgs {
     void *out;
     const int32_t *blocks;
     const int32_t *sched;
+    int groups;
     int sched_wgs, sched_waves;
     int nnz, batches;
     float scale;

@@ -7,7 +7,8 @@
 // workspace so the column pass can attach it to its pairs.
 //
 // Schedule: see bsa.h.  A serial first-fit pass over the groups (one lane)
-// fixes each group's first slot, then all lanes fill the slots.
+// fixes each group's first slot and its partial-tile slots, then all lanes
+// fill the wavefront slots.
 #include "bsa_device.hpp"
 #include "bsa_internal.hpp"
 
@@ -87,46 +88,88 @@ __global__ __launch_bounds__(LB_THREADS) void layout_build_kernel(
 }
 
 // ---- schedule -------------------------------------------------------------
+// Buffer layout (int4 units): [0, groups) per-group meta, then the wavefront slots.
+//   meta[g] = (first slot of part 0, first partial-tile slot or -1, ordinal among split groups or -1, parts)
 
-__device__ __forceinline__ int waves_of_group(int len, int cap, int waves)
+struct GroupPlan {
+    int parts;      // workgroup-sized pieces the group is cut into
+    int len;
+};
+
+__device__ __forceinline__ GroupPlan plan_group(int len, int cap, int waves, int allow_split)
 {
-    int nw = (len + cap - 1) / cap;
+    GroupPlan p;
+    p.len = len;
+    const int span = cap * waves;                       // pairs one workgroup takes at the target chunk size
+    int parts = allow_split ? (len + span - 1) / span : 1;
+    parts = parts < 1 ? 1 : (parts > SCHED_MAX_PARTS ? SCHED_MAX_PARTS : parts);
+    p.parts = parts;
+    return p;
+}
+
+// pairs [lo, hi) of piece t out of n of a range of `len`
+__device__ __forceinline__ int piece_lo(int len, int t, int n) { return (int)(((long long)len * t) / n); }
+
+__device__ __forceinline__ int waves_of_part(int part_len, int cap, int waves)
+{
+    int nw = (part_len + cap - 1) / cap;
     nw = nw < 1 ? 1 : nw;
     return nw > waves ? waves : nw;
 }
 
 __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
-    const int *__restrict__ offsets, int groups, int cap, int waves,
-    int4 *__restrict__ sched, int capacity, int *__restrict__ n_wgs_out, int *__restrict__ first_slot)
+    const int *__restrict__ offsets, int groups, int cap, int waves, int allow_split,
+    int4 *__restrict__ sched, int slot_capacity, int *__restrict__ counts_out)
 {
     __shared__ int total_slots;
     const int tid = (int)threadIdx.x;
-    // first-fit: a team never straddles a workgroup boundary
+    int4 *meta = sched;
+    int4 *slots = sched + groups;
+    // serial first-fit: a team (the waves of one part) never straddles a workgroup boundary
     if (tid == 0) {
-        int pos = 0;
+        int pos = 0, tile_slots = 0, split_groups = 0;
         for (int g = 0; g < groups; ++g) {
-            int nw = waves_of_group(offsets[g + 1] - offsets[g], cap, waves);
-            int in_wg = pos % waves;
-            if (in_wg + nw > waves) pos += waves - in_wg;
-            first_slot[g] = pos;
-            pos += nw;
+            const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split);
+            int first = -1;
+            for (int p = 0; p < gp.parts; ++p) {
+                int plen = piece_lo(gp.len, p + 1, gp.parts) - piece_lo(gp.len, p, gp.parts);
+                int nw = waves_of_part(plen, cap, waves);
+                int in_wg = pos % waves;
+                if (in_wg + nw > waves) pos += waves - in_wg;
+                if (p == 0) first = pos;
+                pos += nw;
+            }
+            const bool split = gp.parts > 1;
+            meta[g] = make_int4(first, split ? tile_slots : -1, split ? split_groups : -1, gp.parts);
+            if (split) { tile_slots += gp.parts; split_groups += 1; }
         }
         int n_wgs = (pos + waves - 1) / waves;
         total_slots = n_wgs * waves;
-        n_wgs_out[0] = n_wgs;
+        counts_out[0] = n_wgs;
+        counts_out[1] = tile_slots;
+        counts_out[2] = split_groups;
+        counts_out[3] = pos;
     }
     __syncthreads();
-    const int slots = total_slots < capacity ? total_slots : capacity;
-    for (int s = tid; s < slots; s += LB_THREADS) sched[s] = make_int4(-1, 0, 0, 0);
+    const int n_slots = total_slots < slot_capacity ? total_slots : slot_capacity;
+    for (int s = tid; s < n_slots; s += LB_THREADS) slots[s] = make_int4(-1, 0, 0, 0);
     __syncthreads();
     for (int g = tid; g < groups; g += LB_THREADS) {
-        int lo = offsets[g], len = offsets[g + 1] - lo;
-        int nw = waves_of_group(len, cap, waves);
-        int s0 = first_slot[g];
-        for (int t = 0; t < nw; ++t) {
-            int b = lo + (int)(((long long)len * t) / nw);
-            int e = lo + (int)(((long long)len * (t + 1)) / nw);
-            if (s0 + t < capacity) sched[s0 + t] = make_int4(g, b, e, (s0 % waves) | (nw << 8));
+        const int lo = offsets[g];
+        const GroupPlan gp = plan_group(offsets[g + 1] - lo, cap, waves, allow_split);
+        int pos = meta[g].x;
+        for (int p = 0; p < gp.parts; ++p) {
+            const int pb = piece_lo(gp.len, p, gp.parts), pe = piece_lo(gp.len, p + 1, gp.parts);
+            const int plen = pe - pb;
+            const int nw = waves_of_part(plen, cap, waves);
+            const int in_wg = pos % waves;
+            if (in_wg + nw > waves) pos += waves - in_wg;
+            for (int t = 0; t < nw; ++t) {
+                const int b = lo + pb + piece_lo(plen, t, nw), e = lo + pb + piece_lo(plen, t + 1, nw);
+                if (pos + t < slot_capacity)
+                    slots[pos + t] = make_int4(g, b, e, sched_team_word(pos % waves, nw, p, gp.parts));
+            }
+            pos += nw;
         }
     }
 }
@@ -144,14 +187,12 @@ hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_b
 }
 
 hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                                 int32_t *sched, int64_t capacity, int32_t *n_wgs_out,
-                                 hipStream_t stream)
+                                 int allow_split, int32_t *sched, int64_t capacity,
+                                 int32_t *counts_out, hipStream_t stream)
 {
-    // the tail of the buffer parks the first slot of every group
-    int64_t slot_capacity = capacity - (groups + 3) / 4;
-    int *first_slot = sched + 4 * slot_capacity;
-    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, (int4 *)sched,
-                                                       (int)slot_capacity, n_wgs_out, first_slot);
+    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, allow_split,
+                                                       (int4 *)sched, (int)(capacity - groups),
+                                                       counts_out);
     return hipGetLastError();
 }
 

@@ -241,7 +241,7 @@ __device__ __forceinline__ bool team_reduce(f16v (&acc)[2], const SchedEntry &e,
                                             unsigned char *lds_raw)
 {
     const int l = lane_id();
-    const int slot0 = e.team & 0xFF, nw = e.team >> 8;
+    const int slot0 = e.first_wave(), nw = e.team_waves();
     const bool active = e.group >= 0;
     const bool leader = active && w == slot0;
     float *mine = reinterpret_cast<float *>(lds_raw + (size_t)w * GW_LDS_PER_WAVE);
@@ -265,10 +265,58 @@ __device__ __forceinline__ bool team_reduce(f16v (&acc)[2], const SchedEntry &e,
     return leader;
 }
 
+// Split groups: every part parks its fp32 partial tile in the workspace and bumps
+// the group's counter; the part that arrives last adds the tiles up in part order
+// (so the sum does not depend on arrival order), resets the counter and returns
+// true: it stores the result.  Tiles and counters are read and written with
+// agent-scope accesses that go to L2, and all parts of a (batch, group) run on one
+// XCD, so no cache write-back is needed; the wait on vmcnt orders tile before counter.
+struct SplitWorkspace {
+    int *counters;     // [batches][strips][split_groups], zero between launches
+    float *tiles;      // [batches][strips][tile_slots][2048]
+    int tile_slots, split_groups;
+};
+
+__device__ __forceinline__ bool split_combine(f16v (&acc)[2], const SchedEntry &e, const SchedGroup &sg,
+                                              const SplitWorkspace &ws, int batch)
+{
+    const int l = lane_id();
+    const int parts = e.parts();
+    const size_t cell = (size_t)batch * gridDim.y + blockIdx.y;
+    float *tile0 = ws.tiles + (cell * ws.tile_slots + sg.tile_slot) * 2048;
+    float *mine = tile0 + (size_t)e.part() * 2048;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            __hip_atomic_store(mine + (t * 16 + v) * WAVE + l, acc[t][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    int *counter = ws.counters + cell * ws.split_groups + sg.split_index;
+    int old = 0;
+    if (l == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __builtin_amdgcn_readfirstlane(old);
+    if (old != parts - 1) return false;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+    for (int p = 0; p < parts; ++p) {
+        const float *src = tile0 + (size_t)p * 2048;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                acc[t][v] += __hip_atomic_load(src + (t * 16 + v) * WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
 template <bool S_KC, bool D_KC, bool DSD, int DEPTH>
 __global__ __launch_bounds__(512) void gw_f16_kernel(
     const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
-    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
+    const SchedEntry *__restrict__ sched, SplitWorkspace ws,
     int n_swg, int batches, int nnz, int DN, int KT, int XT)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -361,7 +409,8 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
         }
     }
 
-    if (team_reduce(acc, e, w, lds_raw)) {
+    if (team_reduce(acc, e, w, lds_raw) &&
+        (e.parts() <= 1 || split_combine(acc, e, sched_groups[e.group], ws, batch))) {
         half_t *ob = out + (size_t)batch * XT * DN;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -379,7 +428,8 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
 template <bool S_KC, bool D_KC, bool DSD>
 __global__ __launch_bounds__(512) void gw_f32_kernel(
     const float *__restrict__ sp, const float *__restrict__ dn, float *__restrict__ out,
-    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
+    const SchedEntry *__restrict__ sched, SplitWorkspace ws,
     int n_swg, int batches, int nnz, int DN, int KT, int XT)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -419,7 +469,8 @@ __global__ __launch_bounds__(512) void gw_f32_kernel(
             }
         }
     }
-    if (team_reduce(acc, e, w, lds_raw)) {
+    if (team_reduce(acc, e, w, lds_raw) &&
+        (e.parts() <= 1 || split_combine(acc, e, sched_groups[e.group], ws, batch))) {
         float *ob = out + (size_t)batch * XT * DN;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -431,6 +482,8 @@ __global__ __launch_bounds__(512) void gw_f32_kernel(
 // launchers
 // ---------------------------------------------------------------------------
 static inline unsigned grid_x(int n_swg, int batches) { return 8u * (unsigned)n_swg * (unsigned)((batches + 7) / 8); }
+static inline const SchedGroup *sched_groups(const MatmulArgs &p) { return (const SchedGroup *)p.sched; }
+static inline const SchedEntry *sched_slots(const MatmulArgs &p) { return (const SchedEntry *)p.sched + p.groups; }
 
 template <bool A_KC, bool B_KC>
 static hipError_t launch_sdd_f16(const MatmulArgs &p, hipStream_t st)
@@ -438,7 +491,7 @@ static hipError_t launch_sdd_f16(const MatmulArgs &p, hipStream_t st)
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
     size_t lds = (size_t)p.sched_waves * SDD_LDS_PER_WAVE;
 #define BSA_SDD_ARGS (const half_t *)p.a, (const half_t *)p.b, (half_t *)p.c, (const BlockDesc *)p.blocks, \
-                     (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K
+                     sched_slots(p), p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K
     switch (p.K / BS) {
         case 1: sdd_f16_kernel<A_KC, B_KC, 1><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
         case 2: sdd_f16_kernel<A_KC, B_KC, 2><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
@@ -456,7 +509,7 @@ static hipError_t launch_sdd_f32(const MatmulArgs &p, hipStream_t st)
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
     sdd_f32_kernel<A_KC, B_KC><<<grid, block, 0, st>>>(
         (const float *)p.a, (const float *)p.b, (float *)p.c, (const BlockDesc *)p.blocks,
-        (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K);
+        sched_slots(p), p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K);
     return hipGetLastError();
 }
 
@@ -479,15 +532,33 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
 {
     dim3 grid(grid_x(p.sched_wgs, p.batches), (unsigned)((DN + 63) / 64)), block(64 * p.sched_waves);
     size_t lds = (size_t)p.sched_waves * GW_LDS_PER_WAVE;
+    // workspace: counters of every (batch, strip, split group), then the partial tiles
+    SplitWorkspace ws;
+    ws.tile_slots = p.tile_slots;
+    ws.split_groups = p.split_groups;
+    ws.counters = (int *)p.workspace;
+    ws.tiles = (float *)((char *)p.workspace + gw_counter_bytes(p.split_groups, p.batches, DN));
     if (dtype == BSA_F16)
         gw_f16_kernel<S_KC, D_KC, DSD, 3><<<grid, block, lds, st>>>(
             (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
-            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
     else
         gw_f32_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(
             (const float *)sp, (const float *)dn, (float *)p.c, (const BlockDesc *)p.blocks,
-            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
     return hipGetLastError();
+}
+
+size_t gw_counter_bytes(int split_groups, int batches, int free_dim)
+{
+    size_t n = (size_t)split_groups * batches * ((free_dim + 63) / 64) * sizeof(int);
+    return (n + 255) / 256 * 256;
+}
+
+size_t gw_workspace_bytes(int tile_slots, int split_groups, int batches, int free_dim)
+{
+    return gw_counter_bytes(split_groups, batches, free_dim) +
+           (size_t)tile_slots * batches * ((free_dim + 63) / 64) * 2048 * sizeof(float);
 }
 
 hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream_t st)

@@ -209,7 +209,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
     for (int q = 0; q < NQ; ++q) s[q] = row_allreduce<LPR>(s[q], AddOp());
 
     // team exchange of (max, sum) per element row
-    const int slot0 = e.team & 0xFF, nw = e.team >> 8;
+    const int slot0 = e.first_wave(), nw = e.team_waves();
     if (active && (l % LPR) == 0) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) stats[w][row0 + q * ROWS_PER_Q] = make_float2(m[q], s[q]);
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
 #pragma unroll
     for (int q = 0; q < NQ; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
 
-    const int slot0 = e.team & 0xFF, nw = e.team >> 8;
+    const int slot0 = e.first_wave(), nw = e.team_waves();
     if (active && (l % LPR) == 0) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) dots[w][row0 + q * ROWS_PER_Q] = dot[q];
@@ -401,11 +401,11 @@ hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t s
     if (dtype == BSA_F16)
         softmax_fwd_kernel<half_t, 8><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (half_t *)p.out, (const BlockDesc *)p.blocks,
-            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
+            (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
     else
         softmax_fwd_kernel<float, 4><<<grid, block, 0, st>>>(
             (const float *)p.x, (float *)p.out, (const BlockDesc *)p.blocks,
-            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
+            (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
     return hipGetLastError();
 }
 
@@ -415,11 +415,11 @@ hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t 
     if (dtype == BSA_F16)
         softmax_bwd_kernel<half_t, 4><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (const half_t *)p.dy, (half_t *)p.out, (const BlockDesc *)p.blocks,
-            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.scale);
+            (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     else
         softmax_bwd_kernel<float, 2><<<grid, block, 0, st>>>(
             (const float *)p.x, (const float *)p.dy, (float *)p.out, (const BlockDesc *)p.blocks,
-            (const SchedEntry *)p.sched, p.sched_wgs, p.batches, p.nnz, p.scale);
+            (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     return hipGetLastError();
 }
 

@@ -21,18 +21,33 @@ _DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
 class Schedule:
     """Device-resident wavefront schedule of one offset table."""
 
-    def __init__(self, offsets: torch.Tensor, nnz: int, cap: int, waves: int):
+    def __init__(self, offsets: torch.Tensor, nnz: int, cap: int, waves: int, allow_split: bool = True):
         groups = offsets.numel() - 1
         capacity = _k.lib.bsa_schedule_capacity(groups, nnz, cap, waves)
         self.table = torch.empty(4 * capacity, dtype=torch.int32, device=offsets.device)
-        n_wgs = torch.empty(1, dtype=torch.int32, device=offsets.device)
+        counts = torch.empty(4, dtype=torch.int32, device=offsets.device)
         with torch.cuda.device(offsets.device):
-            _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves,
-                                               self.table.data_ptr(), capacity, n_wgs.data_ptr(),
+            _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves, int(allow_split),
+                                               self.table.data_ptr(), capacity, counts.data_ptr(),
                                                _k.current_stream()))
-        self.workgroups = int(n_wgs.item())
+        self.workgroups, self.tile_slots, self.split_groups, self.slots = (int(v) for v in counts.tolist())
+        self.groups = groups
         self.waves = waves
         self.cap = cap
+        self._workspaces = {}
+
+    def workspace(self, mode: int, batches: int, size_m: int, size_n: int, stream: int):
+        """Zeroed scratch for split groups, one per (shape, stream): launches on one stream run in
+        order and each leaves the buffer zero again; launches on different streams may overlap."""
+        need = _k.lib.bsa_matmul_workspace_bytes(mode, self.tile_slots, self.split_groups, batches, size_m, size_n)
+        if need == 0:
+            return None, 0
+        key = (mode, batches, size_m, size_n, stream)
+        ws = self._workspaces.get(key)
+        if ws is None:
+            ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
+            self._workspaces[key] = ws
+        return ws, need
 
 
 def schedule_for(layout, kind):
@@ -46,6 +61,11 @@ def schedule_for(layout, kind):
     if kind not in cache:
         cache[kind] = Schedule(offsets, blocks.numel() // 2, *kind)
     return cache[kind]
+
+
+def _softmax_schedule(layout):
+    cap, waves = SCHEDULE_SOFTMAX
+    return schedule_for(layout, (cap, waves, False))
 
 
 def _check_layout(layout, name):
@@ -115,12 +135,15 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
 
     sched = schedule_for(layout, SCHEDULE_SDD if mode == "sdd" else SCHEDULE_GROUP_WALK)
     with torch.cuda.device(a.device):
+        stream = _k.current_stream()
+        ws, ws_bytes = sched.workspace(_k.MODES[mode], batches, size_m, size_n, stream)
         _k.check(_k.lib.bsa_matmul(
             _k.MODES[mode], _DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), c.data_ptr(),
             layout[0].data_ptr(), layout[1].data_ptr(), layout[1].numel() - 1,
-            sched.table.data_ptr(), sched.workgroups, sched.waves,
+            sched.table.data_ptr(), sched.workgroups, sched.waves, sched.tile_slots, sched.split_groups,
+            ws.data_ptr() if ws is not None else None, ws_bytes,
             mask_rows, mask_cols, num_blocks, batches, size_m, size_n, size_k,
-            int(trans_a), int(trans_b), _k.current_stream()))
+            int(trans_a), int(trans_b), stream))
     return c
 
 
@@ -148,7 +171,7 @@ def sparse_softmax_forward(x, row_blocks, row_table, scale=1.0, causal=False, co
     y = torch.empty_like(x)
     if nnz == 0 or x.numel() == 0:
         return y
-    sched = schedule_for(row_layout, SCHEDULE_SOFTMAX)
+    sched = _softmax_schedule(row_layout)
     with torch.cuda.device(x.device):
         _k.check(_k.lib.bsa_softmax_forward(
             _DTYPES[x.dtype], x.data_ptr(), y.data_ptr(), row_blocks.data_ptr(), row_table.data_ptr(),
@@ -168,7 +191,7 @@ def sparse_softmax_backward(y, dy, row_blocks, row_table, scale=1.0, col_layout=
     dx = torch.empty_like(y)
     if nnz == 0 or y.numel() == 0:
         return dx
-    sched = schedule_for(row_layout, SCHEDULE_SOFTMAX)
+    sched = _softmax_schedule(row_layout)
     with torch.cuda.device(y.device):
         _k.check(_k.lib.bsa_softmax_backward(
             _DTYPES[y.dtype], y.data_ptr(), dy.data_ptr(), dx.data_ptr(), row_blocks.data_ptr(),

@@ -21,11 +21,16 @@
  *   offsets  int32[G+1]    first pair of every group: G = mask rows for the
  *                          row layout, mask columns for the column layout
  *
- * Schedule format (new in this build): int32[4] per wavefront slot,
- * (group, first pair, one-past-last pair, team), team = (slot of the team's
- * first wave inside its workgroup) | (waves in the team << 8); group = -1
- * marks an unused slot.  A workgroup owns `waves` consecutive slots; all waves
- * that share a group sit in one workgroup so they can reduce through LDS.
+ * Schedule format (new in this build), int32[4] records:
+ *   [0, groups)   one per group: (first slot, first partial-tile slot or -1,
+ *                 ordinal among the split groups or -1, parts)
+ *   then one per wavefront slot: (group, first pair, one-past-last pair, team),
+ *                 team = first wave of the team inside its workgroup (bits 0-3)
+ *                 | waves in the team (4-7) | part (8-19) | parts (20-31);
+ *                 group = -1 marks an unused slot.
+ * A workgroup owns `waves` consecutive slots.  A group longer than cap * waves
+ * pairs is cut into parts; the waves of one part (a team) sit in one workgroup
+ * and reduce through LDS, the parts of a group meet in a workspace.
  */
 #ifndef BSA_H_
 #define BSA_H_
@@ -76,18 +81,21 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
 
 /* ---- wavefront schedule -------------------------------------------------
  * Splits every group of a table into chunks of about `cap` pairs, one chunk
- * per wavefront, and packs the wavefronts of a group into one workgroup of
- * `waves` wavefronts (a group longer than cap*waves gets longer chunks).
+ * per wavefront, and packs the wavefronts into workgroups of `waves`
+ * wavefronts.  A group longer than cap * waves pairs is cut into parts of at
+ * most that many pairs when `allow_split` != 0 (matmul), and gets longer
+ * chunks otherwise (softmax, whose rows cannot be split across workgroups).
  * Empty groups get one wavefront with an empty chunk (it writes the zeros).
  * No counterpart in the reference, whose grids are (nnz, B) and
  * (B, M/32, N/32) (sparse/native/sparse_smm_gpu.cu:278-279).
  *   sched        device int32[4 * bsa_schedule_capacity(...)]
- *   n_wgs_out    device int32[1]: workgroups the schedule uses
+ *   counts_out   device int32[4]: workgroups the schedule uses, partial-tile
+ *                slots, split groups, wavefront slots in use
  */
 int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves);
 int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                       int32_t *sched, int64_t capacity, int32_t *n_wgs_out,
-                       void *stream);
+                       int allow_split, int32_t *sched, int64_t capacity,
+                       int32_t *counts_out, void *stream);
 
 /* ---- block-sparse matmul -----------------------------------------------
  * Replaces sparse_matmul's launch half: sparse_smm_32x32x32_kernel_wrapper and
@@ -106,11 +114,21 @@ int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
  *   M, N, K are the dims of op(a) (M x K) and op(b) (K x N); every dim that
  *   runs along the sparse matrix must equal 32 * mask_rows / 32 * mask_cols
  *   (after the transpose), the free dense dim must be a multiple of 32.
+ *   sched_tile_slots / sched_split_groups are counts_out[1] / [2] of the
+ *   schedule.  DSD and DDS with split groups need a workspace of
+ *   bsa_matmul_workspace_bytes(...) bytes that is ZERO before its first use;
+ *   every launch leaves it zero again, so it can be reused by later launches
+ *   on the same stream (launches that overlap in time need separate ones).
+ *   SDD takes no workspace (null, 0).
  * fp16 accumulates in fp32.  Empty groups give zero rows / columns.
  */
+size_t bsa_matmul_workspace_bytes(int mode, int sched_tile_slots, int sched_split_groups,
+                                  int batches, int M, int N);
 int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
                const int32_t *blocks, const int32_t *offsets, int groups,
                const int32_t *sched, int sched_wgs, int sched_waves,
+               int sched_tile_slots, int sched_split_groups,
+               void *workspace, size_t workspace_bytes,
                int mask_rows, int mask_cols, int nnz, int batches,
                int M, int N, int K, int tr_a, int tr_b, void *stream);
 

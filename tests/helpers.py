@@ -35,6 +35,11 @@ def mask_zoo():
     long_row[3, ::7] = 1
     long_row[:, 2] = 1
     zoo.append(("long_row_5x40", long_row))
+    long_col = np.zeros((70, 3), dtype=np.int64)
+    long_col[:, 1] = 1          # one column of 70 blocks: cut into parts that meet in the workspace
+    long_col[::9, 0] = 1
+    long_col[5, 2] = 1
+    zoo.append(("long_col_70x3", long_col))
     return zoo
 
 

@@ -48,9 +48,10 @@ P = 0x1000  # any non-null address: validation fails before anything is derefere
 
 
 def _matmul(k, mode=0, dtype=1, a=P, b=P, c=P, blocks=P, offs=P, groups=4, sched=P, wgs=1, waves=4,
+            tiles=0, splits=0, ws=None, ws_bytes=0,
             R=4, C=4, nnz=5, batches=1, M=128, N=128, K=64, ta=0, tb=1):
-    return k.lib.bsa_matmul(mode, dtype, a, b, c, blocks, offs, groups, sched, wgs, waves, R, C, nnz,
-                            batches, M, N, K, ta, tb, None)
+    return k.lib.bsa_matmul(mode, dtype, a, b, c, blocks, offs, groups, sched, wgs, waves, tiles, splits,
+                            ws, ws_bytes, R, C, nnz, batches, M, N, K, ta, tb, None)
 
 
 @pytest.mark.parametrize("kw,needle", [
@@ -68,6 +69,9 @@ def _matmul(k, mode=0, dtype=1, a=P, b=P, c=P, blocks=P, offs=P, groups=4, sched
     (dict(mode=1, ta=0, tb=0, M=128, K=96, N=64), "op(sparse a)"),
     (dict(mode=2, ta=0, tb=0, M=64, K=96, N=128), "op(sparse b)"),
     (dict(R=0), "mask shape"),
+    (dict(tiles=3, splits=0), "inconsistent"),
+    (dict(mode=1, ta=0, tb=0, M=128, K=128, N=64, tiles=4, splits=2), "workspace"),
+    (dict(mode=1, ta=0, tb=0, M=128, K=128, N=64, tiles=4, splits=2, ws=P, ws_bytes=100), "workspace"),
 ])
 def test_matmul_validation(k, kw, needle):
     rc = _matmul(k, **kw)
@@ -79,11 +83,15 @@ def test_other_entry_points_validate(k):
     assert k.lib.bsa_layout_build(None, 4, 4, P, P, P, P, P, P, None) == -1
     assert k.lib.bsa_layout_build(P, 40000, 4, P, P, P, P, P, P, None) == -1
     assert "32767" in k.lib.bsa_last_error().decode()
-    assert k.lib.bsa_schedule_build(P, 4, 0, 4, P, 100, P, None) == -1
-    assert k.lib.bsa_schedule_build(P, 4, 4, 4, P, 3, P, None) == -1
+    assert k.lib.bsa_schedule_build(P, 4, 0, 4, 1, P, 100, P, None) == -1
+    assert k.lib.bsa_schedule_build(P, 4, 4, 4, 1, P, 3, P, None) == -1
     assert "capacity" in k.lib.bsa_last_error().decode()
     assert k.lib.bsa_softmax_forward(3, P, P, P, P, P, 1, 4, 4, 4, 5, 1, 1.0, 0, None) == -3
     assert k.lib.bsa_softmax_forward(1, P, None, P, P, P, 1, 4, 4, 4, 5, 1, 1.0, 0, None) == -1
     assert k.lib.bsa_softmax_backward(1, P, P, P, P, P, P, 1, 4, 4, 4, 5, 0, 1.0, None) == -1
     assert k.lib.bsa_layout_workspace_bytes(4, 8) == 128
-    assert k.lib.bsa_schedule_capacity(4, 5, 4, 8) >= 2 * (4 + 1) + 8 + 1
+    assert k.lib.bsa_schedule_capacity(4, 5, 4, 8) >= 2 * (4 + 1) + 8 + 4
+    # workspace: counters (padded to 256 bytes) + one 8 KB fp32 tile per slot, batch and 64-wide strip
+    assert k.lib.bsa_matmul_workspace_bytes(0, 4, 2, 3, 128, 128) == 0
+    assert k.lib.bsa_matmul_workspace_bytes(1, 0, 0, 3, 128, 128) == 0
+    assert k.lib.bsa_matmul_workspace_bytes(1, 4, 2, 3, 128, 128) == 256 + 4 * 3 * 2 * 8192

@@ -71,35 +71,57 @@ def test_golden_tables_on_device():
 
 
 @pytest.mark.parametrize("name,mask", _more_masks())
-@pytest.mark.parametrize("cap,waves", [(4, 8), (1, 4), (16, 2), (3, 1)])
-def test_schedule_covers_every_pair_once(name, mask, cap, waves):
+@pytest.mark.parametrize("cap,waves,split", [(4, 8, True), (1, 4, True), (16, 2, True), (3, 1, True),
+                                             (4, 8, False), (2, 2, False)])
+def test_schedule_covers_every_pair_once(name, mask, cap, waves, split):
     from sparse import _ops
     mask = np.asarray(mask)
     L = _layout(mask)
     for layout in (L.row_layout, L.col_layout):
         offs = layout[1].cpu().numpy()
         groups = len(offs) - 1
-        s = _ops.Schedule(layout[1], layout[0].numel() // 2, cap, waves)
-        tab = s.table.cpu().numpy()[: 4 * s.workgroups * waves].reshape(-1, 4)
+        s = _ops.Schedule(layout[1], layout[0].numel() // 2, cap, waves, split)
+        raw = s.table.cpu().numpy().reshape(-1, 4)
+        meta = raw[:groups]
+        tab = raw[groups: groups + s.workgroups * waves]
+        assert s.slots <= s.workgroups * waves
         seen = np.zeros(max(int(offs[-1]), 1), dtype=np.int64)
-        group_seen = np.zeros(groups, dtype=np.int64)
+        parts_seen = [set() for _ in range(groups)]
+        tile_slots = split_groups = 0
         for slot, (g, b, e, team) in enumerate(tab):
             if g < 0:
                 continue
-            first, nw = team & 0xFF, team >> 8
+            team = int(team) & 0xFFFFFFFF
+            first, nw, part, parts = team & 0xF, (team >> 4) & 0xF, (team >> 8) & 0xFFF, team >> 20
             wg, in_wg = divmod(slot, waves)
             assert 0 <= g < groups and offs[g] <= b <= e <= offs[g + 1]
-            assert first <= in_wg < first + nw <= waves            # team sits inside one workgroup
+            assert first <= in_wg < first + nw <= waves            # a team sits inside one workgroup
+            assert parts == meta[g][3] and 0 <= part < parts
             leader = tab[wg * waves + first]
-            assert leader[0] == g                                   # same group as its leader
+            assert leader[0] == g and leader[3] == tab[slot][3]
             seen[b:e] += 1
             if in_wg == first:
-                group_seen[g] += 1
-                # chunks of a team are consecutive and tile the group
+                assert part not in parts_seen[g]
+                parts_seen[g].add(part)
                 chunks = tab[wg * waves + first: wg * waves + first + nw]
-                assert chunks[0][1] == offs[g] and chunks[-1][2] == offs[g + 1]
-                assert all(chunks[i][2] == chunks[i + 1][1] for i in range(nw - 1))
-                length = offs[g + 1] - offs[g]
-                assert nw == min(max(-(-length // cap), 1), waves)
+                assert all(chunks[i][2] == chunks[i + 1][1] for i in range(nw - 1))   # consecutive
+                plen = chunks[-1][2] - chunks[0][1]
+                assert nw == min(max(-(-plen // cap), 1), waves)
+                if split:
+                    assert plen <= cap * waves
+                if part == 0:
+                    assert chunks[0][1] == offs[g] and meta[g][0] == slot
+                if part == parts - 1:
+                    assert chunks[-1][2] == offs[g + 1]
         assert np.all(seen[: int(offs[-1])] == 1)
-        assert np.all(group_seen == 1)                              # empty groups get a slot too
+        for g in range(groups):
+            length = offs[g + 1] - offs[g]
+            want = max(-(-length // (cap * waves)), 1) if split else 1
+            assert parts_seen[g] == set(range(want)), (g, parts_seen[g], want)   # empty groups get a slot too
+            if want > 1:
+                assert meta[g][1] == tile_slots and meta[g][2] == split_groups
+                tile_slots += want
+                split_groups += 1
+            else:
+                assert meta[g][1] == -1 and meta[g][2] == -1
+        assert (s.tile_slots, s.split_groups) == (tile_slots, split_groups)

@@ -30,7 +30,7 @@ def _run(mode, mask, free, ta, tb, dtype, batch=(2,), seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("mode,ta,tb", VARIANTS)
-@pytest.mark.parametrize("name", ["known3x3", "empty_row_col_6x5", "long_row_5x40"])
+@pytest.mark.parametrize("name", ["known3x3", "empty_row_col_6x5", "long_row_5x40", "long_col_70x3"])
 def test_all_variants(name, mode, ta, tb, dtype):
     err = _run(mode, ZOO[name], 64, ta, tb, dtype)
     assert err <= tol_of(dtype), err
@@ -57,6 +57,35 @@ def test_edge_layouts(name, mode, dtype):
 def test_multiple_batch_dims_and_many_batches(mode, ta, tb):
     assert _run(mode, ZOO["known3x3"], 64, ta, tb, torch.float16, batch=(2, 3)) <= tol_of(torch.float16)
     assert _run(mode, ZOO["known3x3"], 64, ta, tb, torch.float32, batch=(19,)) <= tol_of(torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("mode,ta,tb", [("dsd", False, False), ("dsd", True, False), ("dds", False, False), ("dds", False, True)])
+def test_split_groups_reuse_their_workspace(mode, ta, tb, dtype):
+    """Groups longer than one workgroup's span are cut into parts that meet in a workspace the
+    library leaves zeroed: repeated calls, three 64-wide strips, several batches."""
+    import sparse
+    from sparse import _ops
+    old = _ops.SCHEDULE_GROUP_WALK
+    try:
+        for sched in ((2, 2), (4, 8), (3, 1)):
+            _ops.SCHEDULE_GROUP_WALK = sched
+            for name in ("long_row_5x40", "long_col_70x3"):
+                errs = [_run(mode, ZOO[name], 160, ta, tb, dtype, batch=(3,), seed=s) for s in range(3)]
+                assert max(errs) <= tol_of(dtype), (sched, name, errs)
+    finally:
+        _ops.SCHEDULE_GROUP_WALK = old
+
+
+def test_split_result_is_deterministic():
+    import sparse
+    mask = np.asarray(ZOO["long_col_70x3"])
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(4, 64, 70 * 32, generator=g).half().cuda()
+    s = torch.randn(4, L.num_blocks, 32, 32, generator=g).half().cuda()
+    outs = [sparse.matmul(a, s, "dds", L) for _ in range(5)]
+    assert all(torch.equal(outs[0], o) for o in outs[1:])
 
 
 def test_empty_mask_gives_zeros():
