@@ -57,6 +57,36 @@ struct SchedGroup {
     int parts;
 };
 
+__device__ __forceinline__ int lane_id();
+
+// Up to 64 consecutive pairs of the block table, fetched with ONE vector load (lane t
+// keeps pair first + t) and handed out with v_readlane.  A scalar load of blocks[p]
+// inside the loop would put a full memory round trip on the critical path of every
+// block; this way the walk over a chunk touches the table once.
+struct DescWindow {
+    int idx, pos, first;
+    __device__ __forceinline__ void fetch(const BlockDesc *blocks, int begin, int end)
+    {
+        first = begin;
+        int t = begin + (int)(threadIdx.x & 63u);
+        idx = 0;
+        pos = 0;
+        if (t < end) {
+            const BlockDesc d = blocks[t];
+            idx = d.idx;
+            pos = d.pos;
+        }
+    }
+    // p must be uniform across the wave and inside [first, first + 64)
+    __device__ __forceinline__ BlockDesc get(int p) const
+    {
+        BlockDesc d;
+        d.idx = __builtin_amdgcn_readlane(idx, p - first);
+        d.pos = __builtin_amdgcn_readlane(pos, p - first);
+        return d;
+    }
+};
+
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63u); }
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 

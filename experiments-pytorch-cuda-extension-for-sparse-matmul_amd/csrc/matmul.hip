@@ -26,9 +26,40 @@
 
 namespace bsa {
 
+#ifdef BSA_TRACE
+// Debug builds only: per-wave (start, end, hardware id, work) records for timeline studies.
+__device__ unsigned long long *g_trace = nullptr;
+__device__ __forceinline__ void trace_wave(const unsigned long long (&t)[5], int batch, int group, int nblocks)
+{
+    if (g_trace == nullptr || lane_id() != 0) return;
+    unsigned long long t1 = wall_clock64();
+    unsigned hw = __builtin_amdgcn_s_getreg((4) | (0 << 6) | (31 << 11));
+    unsigned xcc = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (31 << 11));
+    unsigned long long i = atomicAdd(g_trace, 1ull);
+    unsigned long long *r = g_trace + 1 + 8 * i;
+    r[0] = t[0]; r[1] = t1; r[2] = ((unsigned long long)xcc << 32) | hw;
+    r[3] = ((unsigned long long)batch << 40) | ((unsigned long long)group << 16) | (unsigned)nblocks;
+    r[4] = t[1]; r[5] = t[2]; r[6] = t[3]; r[7] = t[4];
+}
+#define BSA_TRACE_MARK(i) { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); trace_t[i] = wall_clock64(); }
+#define BSA_TRACE_MARK_NOWAIT(i) { trace_t[i] = wall_clock64(); }
+__device__ int g_ablate = 0;   // 1: no LDS/MFMA, 2: no dense loads, 4: no sparse loads
+#define BSA_ABLATE(bit) (g_ablate & (bit))
+#define BSA_TRACE_BEGIN unsigned long long trace_t[5]; trace_t[0] = trace_t[1] = trace_t[2] = trace_t[3] = trace_t[4] = wall_clock64();
+#define BSA_TRACE_END(batch, group, n) trace_wave(trace_t, batch, group, n);
+#else
+#define BSA_ABLATE(bit) 0
+#define BSA_TRACE_MARK(i)
+#define BSA_TRACE_MARK_NOWAIT(i)
+#define BSA_TRACE_BEGIN
+#define BSA_TRACE_END(batch, group, n)
+#endif
+
 constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + up to 5 KB), reused for the fp32 partial tile
 constexpr int GW_DENSE_LD = 80;         // halves per row of the staged [k][64] dense tile: 160-byte rows
                                         // put 4 consecutive rows into 4 different 32-byte bank groups
+constexpr int GW_PREFETCH_DEPTH = 2;    // pairs whose operands are in flight per wave: deeper costs 24 VGPRs a
+                                        // stage and did not pay (124 VGPRs = 4 waves per SIMD at depth 2)
 constexpr int SDD_KB_MAX = 4;           // k-blocks (of 32) whose operands stay resident per wave
 constexpr int SDD_LDS_PER_WAVE = 2048 * (1 + SDD_KB_MAX);   // a / result tile + one b tile per k-block
 
@@ -98,36 +129,43 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
         }
         uint4 braw[2][KB][2];
         BlockDesc d[2];
-        d[0] = blocks[e.begin];
+        DescWindow win;
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+            d[0] = win.get(seg);
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) load_b(d[0].col(), kb, braw[0][kb]);
-        for (int p = e.begin; p < e.end; p += 2) {
+            for (int kb = 0; kb < KB; ++kb) load_b(d[0].col(), kb, braw[0][kb]);
+            for (int p = seg; p < seg_end; p += 2) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                if (p + u < e.end) {
-                    if (p + u + 1 < e.end) {
-                        d[u ^ 1] = blocks[p + u + 1];
+                for (int u = 0; u < 2; ++u) {
+                    if (p + u < seg_end) {
+                        if (p + u + 1 < seg_end) {
+                            d[u ^ 1] = win.get(p + u + 1);
 #pragma unroll
-                        for (int kb = 0; kb < KB; ++kb) load_b(d[u ^ 1].col(), kb, braw[u ^ 1][kb]);
+                            for (int kb = 0; kb < KB; ++kb) load_b(d[u ^ 1].col(), kb, braw[u ^ 1][kb]);
+                        }
+                        wave_lds_fence();
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb) put_b(tile_b + kb * BS2, braw[u][kb]);
+                        wave_lds_fence();
+                        f16v acc = {0};
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb) {
+                            acc = mfma_f16(get_b(tile_b + kb * BS2, 0), aop[kb][0], acc);
+                            acc = mfma_f16(get_b(tile_b + kb * BS2, 1), aop[kb][1], acc);
+                        }
+                        store(d[u].idx, acc);
                     }
-                    wave_lds_fence();
-#pragma unroll
-                    for (int kb = 0; kb < KB; ++kb) put_b(tile_b + kb * BS2, braw[u][kb]);
-                    wave_lds_fence();
-                    f16v acc = {0};
-#pragma unroll
-                    for (int kb = 0; kb < KB; ++kb) {
-                        acc = mfma_f16(get_b(tile_b + kb * BS2, 0), aop[kb][0], acc);
-                        acc = mfma_f16(get_b(tile_b + kb * BS2, 1), aop[kb][1], acc);
-                    }
-                    store(d[u].idx, acc);
                 }
             }
         }
     } else {
         const int kbs = K / BS;
+        DescWindow win;
         for (int p = e.begin; p < e.end; ++p) {
-            const BlockDesc d = blocks[p];
+            if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+            const BlockDesc d = win.get(p);
             f16v acc = {0};
             uint4 araw[2], braw[2];
             load_a(0, araw);
@@ -197,8 +235,10 @@ __global__ __launch_bounds__(512) void sdd_f32_kernel(
     float *cb = c + (size_t)batch * nnz * BS2;
     const int r = e.group, kbs = K / BS;
 
+    DescWindow win;
     for (int p = e.begin; p < e.end; ++p) {
-        const BlockDesc d = blocks[p];
+        if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+        const BlockDesc d = win.get(p);
         const int cblk = d.col();
         f16v acc = {0};
         for (int kb = 0; kb < kbs; ++kb) {
@@ -320,6 +360,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     int n_swg, int batches, int nnz, int DN, int KT, int XT)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
+    BSA_TRACE_BEGIN
     int batch, swg;
     if (!map_workgroup(n_swg, batches, batch, swg)) return;   // whole workgroup leaves together
     const int w = wave_id(), l = lane_id();
@@ -337,10 +378,12 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     // every request fully coalesced
     struct Frag { uint4 s[2]; uint4 d0[2]; uint4 d1[2]; };
 
+    DescWindow win;
     auto load = [&](int p, Frag &f) {
-        const BlockDesc d = blocks[p];
+        const BlockDesc d = win.get(p);
         const int kblk = S_KC ? d.col() : d.row();
-        ldg_tile32(spb + (size_t)d.idx * BS2, BS, f.s);
+        if (!BSA_ABLATE(4)) ldg_tile32(spb + (size_t)d.idx * BS2, BS, f.s);
+        if (BSA_ABLATE(2)) return;
         if (D_KC) {          // stored [DN][KT]: two 32 x 32 tiles, rows KT apart
             const half_t *src = dnb + (size_t)y0 * KT + BS * kblk;
             ldg_tile32(src, KT, f.d0);
@@ -364,6 +407,10 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     // DSD: the dense strip feeds the accumulator-register index (perm16), the block the lane index;
     // DDS: the other way round.
     auto compute = [&](const Frag &f) {
+        if (BSA_ABLATE(1)) {
+            acc[0][0] += __uint_as_float(f.s[0].x ^ f.s[1].y ^ f.d0[0].x ^ f.d0[1].y ^ f.d1[0].z ^ f.d1[1].w);
+            return;
+        }
         wave_lds_fence();
         if (S_KC) lds_put_kc<!DSD>(tile_s, f.s);
         else lds_put_ks(tile_s, f.s);
@@ -393,24 +440,33 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
         }
     };
 
+    BSA_TRACE_MARK_NOWAIT(1)
     if (e.group >= 0) {
         Frag fr[DEPTH];
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d)
-            if (e.begin + d < e.end) load(e.begin + d, fr[d]);
-        for (int p = e.begin; p < e.end; p += DEPTH) {
+            for (int d = 0; d < DEPTH; ++d)
+                if (seg + d < seg_end) load(seg + d, fr[d]);
+            BSA_TRACE_MARK_NOWAIT(2)
+            for (int p = seg; p < seg_end; p += DEPTH) {
 #pragma unroll
-            for (int d = 0; d < DEPTH; ++d) {
-                if (p + d < e.end) {
-                    compute(fr[d]);
-                    if (p + d + DEPTH < e.end) load(p + d + DEPTH, fr[d]);
+                for (int d = 0; d < DEPTH; ++d) {
+                    if (p + d < seg_end) {
+                        compute(fr[d]);
+                        if (p + d + DEPTH < seg_end) load(p + d + DEPTH, fr[d]);
+                    }
                 }
             }
         }
     }
 
-    if (team_reduce(acc, e, w, lds_raw) &&
-        (e.parts() <= 1 || split_combine(acc, e, sched_groups[e.group], ws, batch))) {
+    BSA_TRACE_MARK(3)
+    const bool store_it = team_reduce(acc, e, w, lds_raw) &&
+                          (e.parts() <= 1 || split_combine(acc, e, sched_groups[e.group], ws, batch));
+    BSA_TRACE_MARK(4)
+    if (store_it) {
         half_t *ob = out + (size_t)batch * XT * DN;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -423,6 +479,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
             }
         }
     }
+    BSA_TRACE_END(batch, e.group, e.end - e.begin)
 }
 
 template <bool S_KC, bool D_KC, bool DSD>
@@ -445,8 +502,10 @@ __global__ __launch_bounds__(512) void gw_f32_kernel(
 
     f16v acc[2] = {{0}, {0}};
     if (e.group >= 0) {
+        DescWindow win;
         for (int p = e.begin; p < e.end; ++p) {
-            const BlockDesc d = blocks[p];
+            if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+            const BlockDesc d = win.get(p);
             const int kblk = S_KC ? d.col() : d.row();
             float sv[16], dv[2][16];
             ldg_tile_f32<S_KC, !DSD>(spb + (size_t)d.idx * BS2, BS, sv);
@@ -539,7 +598,7 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
     ws.counters = (int *)p.workspace;
     ws.tiles = (float *)((char *)p.workspace + gw_counter_bytes(p.split_groups, p.batches, DN));
     if (dtype == BSA_F16)
-        gw_f16_kernel<S_KC, D_KC, DSD, 3><<<grid, block, lds, st>>>(
+        gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH><<<grid, block, lds, st>>>(
             (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
             sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
     else
@@ -582,5 +641,18 @@ hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream
     return d_kc ? launch_gw_t<false, true, false>(dtype, p.b, p.a, p, DN, KT, XT, st)
                 : launch_gw_t<false, false, false>(dtype, p.b, p.a, p, DN, KT, XT, st);
 }
+
+#ifdef BSA_TRACE
+}  // namespace bsa
+extern "C" int bsa_debug_trace(unsigned long long *buf)
+{
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(bsa::g_trace), &buf, sizeof(buf));
+}
+extern "C" int bsa_debug_ablate(int bits)
+{
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(bsa::g_ablate), &bits, sizeof(bits));
+}
+namespace bsa {
+#endif
 
 }  // namespace bsa

@@ -131,11 +131,13 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
     int bidx[CB], bcol[CB];
     const bool resident = n <= CB;
 
+    DescWindow win;
+    if (active) win.fetch(blocks, e.begin, e.end);
     if (resident) {
 #pragma unroll
         for (int j = 0; j < CB; ++j) {
             if (j < n) {
-                const BlockDesc d = blocks[e.begin + j];
+                const BlockDesc d = win.get(e.begin + j);
                 bidx[j] = d.idx; bcol[j] = d.col();
                 const T *src = xb + (size_t)d.idx * BS2;
 #pragma unroll
@@ -178,7 +180,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
     } else if (active) {
         // streaming pass 1: online max / sum
         for (int p = e.begin; p < e.end; ++p) {
-            const BlockDesc d = blocks[p];
+            if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+            const BlockDesc d = win.get(p);
             const T *src = xb + (size_t)d.idx * BS2;
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
@@ -257,7 +260,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
     } else {
         // streaming pass 2: re-read, normalise, write
         for (int p = e.begin; p < e.end; ++p) {
-            const BlockDesc d = blocks[p];
+            if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+            const BlockDesc d = win.get(p);
             const T *src = xb + (size_t)d.idx * BS2;
             T *dst = yb + (size_t)d.idx * BS2;
 #pragma unroll
@@ -303,11 +307,13 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
     uint4 ry[CB][NQ], rd[CB][NQ];
     int bidx[CB];
     const bool resident = n <= CB;
+    DescWindow win;
+    if (active) win.fetch(blocks, e.begin, e.end);
     if (resident) {
 #pragma unroll
         for (int j = 0; j < CB; ++j) {
             if (j < n) {
-                bidx[j] = blocks[e.begin + j].idx;
+                bidx[j] = win.get(e.begin + j).idx;
                 const size_t o = boff + (size_t)bidx[j] * BS2;
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
@@ -331,7 +337,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
         }
     } else if (active) {
         for (int p = e.begin; p < e.end; ++p) {
-            const size_t o = boff + (size_t)blocks[p].idx * BS2;
+            if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+            const size_t o = boff + (size_t)win.get(p).idx * BS2;
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
                 float a[EPC], b[EPC];
@@ -380,7 +387,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
         }
     } else {
         for (int p = e.begin; p < e.end; ++p) {
-            const size_t o = boff + (size_t)blocks[p].idx * BS2;
+            if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+            const size_t o = boff + (size_t)win.get(p).idx * BS2;
 #pragma unroll
             for (int q = 0; q < NQ; ++q)
                 stg16(dx + o + (l + WAVE * q) * EPC,

@@ -11,9 +11,9 @@ from . import kernel as _k
 
 BLOCK = 32
 # tuning of the wavefront schedules: (target pairs per wavefront, wavefronts per workgroup)
-SCHEDULE_GROUP_WALK = (4, 8)
-SCHEDULE_SDD = (4, 4)
-SCHEDULE_SOFTMAX = (4, 8)
+SCHEDULE_GROUP_WALK = (12, 2)
+SCHEDULE_SDD = (4, 2)
+SCHEDULE_SOFTMAX = (4, 4)
 
 _DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
 
