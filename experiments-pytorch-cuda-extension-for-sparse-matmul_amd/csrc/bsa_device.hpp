@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "lds_index_math.hpp"
+
 namespace bsa {
 
 typedef _Float16 half_t;
@@ -90,12 +92,6 @@ struct DescWindow {
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63u); }
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
-// MFMA 32x32 accumulators give lane (l % 32, h = l / 32) the result rows
-// 8 * (v / 4) + 4 * h + v % 4, v = 0..15.  Feeding the row operand through this
-// permutation makes those 16 values 16 CONSECUTIVE logical indices 16 * h + v,
-// so a lane can store them with two 16-byte (fp16) or four (fp32) writes.
-__device__ __forceinline__ int perm16(int i) { return (i & 3) + 4 * (i >> 3) + 16 * ((i >> 2) & 1); }
-
 // Workgroup -> (batch, schedule workgroup).  Hardware deals consecutive
 // workgroup ids round-robin to the 8 XCDs, each with its own 4 MB L2; batch b
 // is pinned to XCD b % 8 so that its dense operand is fetched into one L2 only.
@@ -130,31 +126,6 @@ __device__ __forceinline__ h4 lds_read_tr16(const half_t *p)
     typedef tr4 __attribute__((address_space(3))) *lds_tr4_ptr;
     tr4 r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_tr4_ptr)(uintptr_t)p);
     return __builtin_bit_cast(h4, r);
-}
-
-// Chunk base (in elements) handed in by source lane quad a = s % 4 of lane
-// group g = lane / 16, for a 32-wide index range: natural order gives result
-// lane l the index l % 32; the permuted order gives it perm16(l % 32).
-template <bool PERMUTED>
-__device__ __forceinline__ int tr_chunk_base(int g, int a)
-{
-    if (PERMUTED) return 8 * (g & 1) + 4 * (a >> 1) + 16 * (a & 1);
-    return 16 * (g & 1) + 4 * a;
-}
-
-// Reads the 8 halves k = 16 * step + 8 * (lane / 32) + 0..7 of one index from a
-// [k][x] tile in LDS with row stride `ld` halves; `x0` is the first column of
-// the 32-wide index range.
-template <bool PERMUTED>
-__device__ __forceinline__ h8 lds_operand_tr(const half_t *tile, int ld, int x0, int step)
-{
-    int l = lane_id();
-    int g = l >> 4, s = l & 15;
-    int k = 16 * step + 8 * (g >> 1) + (s >> 2);
-    int x = x0 + tr_chunk_base<PERMUTED>(g, s & 3);
-    h4 lo = lds_read_tr16(tile + k * ld + x);
-    h4 hi = lds_read_tr16(tile + (k + 4) * ld + x);
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
 __device__ __forceinline__ f16v mfma_f16(h8 a, h8 b, f16v c)

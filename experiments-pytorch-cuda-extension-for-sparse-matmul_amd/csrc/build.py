@@ -9,7 +9,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["api.hip", "layout_build.hip", "matmul.hip", "softmax.hip"]
-HEADERS = ["bsa_device.hpp", "lds_tiles.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
+HEADERS = ["bsa_device.hpp", "lds_tiles.hpp", "lds_index_math.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
 LIB = os.path.join(HERE, "libbsa_hip.so")
 
 FLAGS = [
@@ -40,7 +40,19 @@ def build(force: bool = False, verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed building libbsa_hip.so")
     if verbose and res.stderr.strip():
         sys.stderr.write(res.stderr)
+    build_index_host(verbose)
     return LIB
+
+
+def build_index_host(verbose: bool = False) -> str:
+    """g++ build of the LDS index arithmetic (no GPU code) for the bank-model tests."""
+    out = os.path.join(HERE, "liblds_index.so")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+           os.path.join(HERE, "lds_index_host.cpp"), "-o", out]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return out
 
 
 if __name__ == "__main__":

@@ -1,0 +1,99 @@
+// Pure index arithmetic of the LDS tile layouts and of the MFMA lane maps, usable
+// on the host and on the device.  Kept free of HIP so that the same functions the
+// kernels use can be compiled with g++ and replayed through the LDS bank model
+// (tests/test_lds_bank_model.py).  Units: a "piece" is 16 bytes = 8 halves.
+#pragma once
+
+#if defined(__HIPCC__)
+#define BSA_HD __host__ __device__ __forceinline__
+#else
+#define BSA_HD inline
+#endif
+
+namespace bsa {
+
+// MFMA 32x32 accumulators give lane (l % 32, h = l / 32) the result rows
+// 8 * (v / 4) + 4 * h + v % 4, v = 0..15.  Feeding the row operand through this
+// permutation makes those 16 values 16 CONSECUTIVE logical indices 16 * h + v,
+// so a lane can store them with two 16-byte (fp16) or four (fp32) writes.
+BSA_HD constexpr int perm16(int i) { return (i & 3) + 4 * (i >> 3) + 16 * ((i >> 2) & 1); }
+BSA_HD constexpr int invperm16(int r) { return (r & 3) + 4 * ((r >> 4) & 1) + 8 * ((r >> 2) & 3); }
+
+// Tile stored [index][k] (contraction contiguous), 64-byte rows: 16-byte slot of
+// piece p of row r.  An operand read takes the SAME piece of 16 consecutive rows
+// per 16-lane phase; rows r, r + 4, r + 8, r + 12 start at the same offset of the
+// 256-byte bank window, so the XOR sends them to the four different pieces.  The
+// mask depends on r % 16 only: lanes i and i + 16 of a 32-lane half must use the
+// same banks or the read takes twice as long (measured with lds_bank_probe).
+BSA_HD constexpr int kc_swizzle(int row) { return (row >> 2) & 3; }
+BSA_HD constexpr int kc_slot(int row, int piece) { return row * 4 + (piece ^ kc_swizzle(row)); }
+
+// Tile stored [k][index] (contraction is the slow index), 64-byte rows.  A lane
+// group of a transposing read takes two pieces ({0,1}, {2,3}, {0,2} or {1,3}) of 4
+// consecutive rows; rows k and k + 2 share a bank window and flip both piece bits.
+BSA_HD constexpr int ks_swizzle(int k) { return 3 * ((k >> 1) & 1); }
+BSA_HD constexpr int ks_slot(int k, int piece) { return k * 4 + (piece ^ ks_swizzle(k)); }
+
+// [k][64] dense strip, 128-byte rows (8 pieces): a lane group takes pieces
+// {2m, 2m+1} or {j, j+2} of 4 consecutive rows; the four XOR masks 0, 3, 4, 7 keep
+// both kinds of pairs apart across the rows.
+BSA_HD constexpr int strip_swizzle(int k) { return 3 * (k & 1) + 4 * ((k >> 1) & 1); }
+
+// Column (in halves) that source-lane quad a of lane group g = lane / 16 hands to
+// ds_read_b64_tr_b16 so that result lane l ends up with index l % 32 (natural) or
+// perm16(l % 32) (permuted).
+BSA_HD constexpr int tr_chunk_base(bool permuted, int g, int a)
+{
+    return permuted ? 8 * (g & 1) + 4 * (a >> 1) + 16 * (a & 1) : 16 * (g & 1) + 4 * a;
+}
+
+// ---- byte addresses inside a wave-private tile, per lane ---------------------
+
+// registers -> LDS of a [index][k] tile: piece c = lane + 64 q of the 2 KB tile
+BSA_HD constexpr int put_kc_addr(bool permuted, int lane, int q)
+{
+    int c = lane + 64 * q;
+    int row = permuted ? invperm16(c >> 2) : (c >> 2);
+    return 16 * kc_slot(row, c & 3);
+}
+// LDS -> MFMA operand, k-step `step`
+BSA_HD constexpr int get_kc_addr(int lane, int step) { return 16 * kc_slot(lane & 31, 2 * step + (lane >> 5)); }
+
+BSA_HD constexpr int put_ks_addr(int lane, int q)
+{
+    int c = lane + 64 * q;
+    return 16 * ks_slot(c >> 2, c & 3);
+}
+// address handed to ds_read_b64_tr_b16 (8 bytes per lane); half = 0 for k..k+3, 1 for k+4..k+7
+BSA_HD constexpr int get_ks_addr(bool permuted, int lane, int step, int half)
+{
+    int g = lane >> 4, s = lane & 15;
+    int k = 16 * step + 8 * (g >> 1) + (s >> 2) + 4 * half;
+    int x = tr_chunk_base(permuted, g, s & 3) ^ (8 * ks_swizzle(k));   // k + 4 swizzles alike
+    return 2 * (k * 32 + x);
+}
+
+// [k][64] dense strip (group walk, contraction slow): piece c = lane + 64 q of the 4 KB strip
+BSA_HD constexpr int put_strip_addr(int lane, int q)
+{
+    int c = lane + 64 * q;
+    int k = c >> 3;
+    return 16 * (k * 8 + ((c & 7) ^ strip_swizzle(k)));
+}
+BSA_HD constexpr int get_strip_addr(bool permuted, int lane, int step, int half, int x0)
+{
+    int g = lane >> 4, s = lane & 15;
+    int k = 16 * step + 8 * (g >> 1) + (s >> 2) + 4 * half;   // k + 4 swizzles alike
+    int x = (x0 + tr_chunk_base(permuted, g, s & 3)) ^ (8 * strip_swizzle(k));
+    return 2 * (k * 64 + x);
+}
+
+// result tile (SDD): lane (row = lane % 32, h = lane / 32) parks columns 16 h .. 16 h + 15
+BSA_HD constexpr int put_result_addr(int lane, int j) { return 16 * kc_slot(lane & 31, 2 * (lane >> 5) + j); }
+BSA_HD constexpr int get_linear_addr(int lane, int q)
+{
+    int c = lane + 64 * q;
+    return 16 * kc_slot(c >> 2, c & 3);
+}
+
+}  // namespace bsa

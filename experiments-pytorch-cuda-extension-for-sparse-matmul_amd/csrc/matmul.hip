@@ -55,9 +55,7 @@ __device__ int g_ablate = 0;   // 1: no LDS/MFMA, 2: no dense loads, 4: no spars
 #define BSA_TRACE_END(batch, group, n)
 #endif
 
-constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + up to 5 KB), reused for the fp32 partial tile
-constexpr int GW_DENSE_LD = 80;         // halves per row of the staged [k][64] dense tile: 160-byte rows
-                                        // put 4 consecutive rows into 4 different 32-byte bank groups
+constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + 4 KB), reused for the fp32 partial tile
 constexpr int GW_PREFETCH_DEPTH = 2;    // pairs whose operands are in flight per wave: deeper costs 24 VGPRs a
                                         // stage and did not pay (124 VGPRs = 4 waves per SIMD at depth 2)
 constexpr int SDD_KB_MAX = 4;           // k-blocks (of 32) whose operands stay resident per wave
@@ -418,12 +416,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
             lds_put_kc<DSD>(tile_d, f.d0);
             if (ytiles == 2) lds_put_kc<DSD>(tile_d + BS2, f.d1);
         } else {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                int cidx = l + 64 * q;
-                *reinterpret_cast<uint4 *>(tile_d + (cidx >> 3) * GW_DENSE_LD + 8 * (cidx & 7)) =
-                    q < 2 ? f.d0[q & 1] : f.d1[q & 1];
-            }
+            lds_put_strip(tile_d, f.d0, f.d1);
         }
         wave_lds_fence();
 #pragma unroll
@@ -433,7 +426,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
             for (int t = 0; t < 2; ++t) {
                 if (t < ytiles) {
                     const h8 dop = D_KC ? lds_get_kc(tile_d + t * BS2, s)
-                                        : lds_operand_tr<DSD>(tile_d, GW_DENSE_LD, 32 * t, s);
+                                        : lds_get_strip<DSD>(tile_d, 32 * t, s);
                     acc[t] = DSD ? mfma_f16(dop, sop, acc[t]) : mfma_f16(sop, dop, acc[t]);
                 }
             }
