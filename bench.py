@@ -10,8 +10,9 @@ A step is one pass of the three products over that batch:
 
 `value` = nnz-block TFLOP/s = 3 * 2 * nnz * 32 * 32 * 64 * 16 flop / step time.
 The softmax (scale 1/8, causal) is timed in its own loop and reported in GB/s.
-Operands rotate over several resident sets so that the footprint exceeds the
-256 MB infinity cache and the figures are HBM figures.  Launches are replayed
+Consecutive launches take the next of several resident operand sets, so every
+launch finds its operands in HBM, not in the 256 MB infinity cache (`--sets 1`
+shows the cache-resident figures).  Launches are replayed
 from HIP graphs (the Python call path costs more than a 10 us kernel).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sets S] [--no-cpu]
@@ -34,7 +35,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--sets", type=int, default=4, help="operand sets to rotate over")
+    ap.add_argument("--sets", type=int, default=6,
+                    help="operand sets to rotate over (1 = the same operands every launch, which the 256 MB "
+                         "infinity cache then serves)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     args = ap.parse_args()
@@ -88,27 +91,36 @@ def main():
         err = ((o[:2].float() - ref).abs().max() / ref.abs().max()).item()
         assert err <= 2e-3, f"DSD parity check failed: {err}"
 
-    # plain copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters of a profiler run
-    cal_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    # plain streaming kernel of known size (reads 64 MiB, writes 64 MiB, 16 bytes per lane), run on
+    # cold caches: the yardstick for the FETCH_SIZE / WRITE_SIZE counters of a profiler run
+    cal_src = torch.randn(16 << 20, dtype=torch.float32, device=dev)
     cal_dst = torch.empty_like(cal_src)
-    cal_dst.copy_(cal_src)
-    del cal_src, cal_dst
+    flush = torch.zeros(256 << 20, dtype=torch.float32, device=dev)   # 1 GiB: evicts L2 and the 256 MB MALL
+    flush.add_(1.0)
+    torch.neg(cal_src, out=cal_dst)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst, flush
 
     stream = torch.cuda.Stream()
 
     def make_runner(fn, reps=1):
-        """One callable per operand set; each replays `reps` launches of fn on that set."""
+        """Callables that each run `reps` launches of fn; consecutive launches always take the next
+        operand set, inside a graph as well as from one graph to the next."""
+        with torch.cuda.stream(stream), torch.no_grad():
+            for w in sets:
+                fn(w)                          # build schedules / workspaces outside capture
+            stream.synchronize()
+        n_graphs = len(sets) if reps % len(sets) else 1
         runners = []
-        for w in sets:
+        for gi in range(n_graphs):
+            order = [sets[(gi * reps + i) % len(sets)] for i in range(reps)]
             if args.no_graph:
-                runners.append(lambda w=w: [fn(w) for _ in range(reps)])
+                runners.append(lambda order=order: [fn(w) for w in order])
                 continue
             g = torch.cuda.CUDAGraph()
             with torch.cuda.stream(stream), torch.no_grad():
-                fn(w)                      # warm the caches / schedules outside capture
-                stream.synchronize()
                 with torch.cuda.graph(g, stream=stream):
-                    keep = [fn(w) for _ in range(reps)]
+                    keep = [fn(w) for w in order]
             runners.append(lambda g=g, keep=keep: g.replay())
         return runners
 
@@ -130,7 +142,7 @@ def main():
     value = 3 * flops_one / (step_ms * 1e-3) / 1e12
 
     # per-kernel average launch duration: REPS launches per graph, events around the replays
-    REPS = 10
+    REPS = 2 * len(sets)
     per_op = {}
     for name, fn in ops.items():
         ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS

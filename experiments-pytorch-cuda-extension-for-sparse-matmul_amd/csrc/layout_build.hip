@@ -92,14 +92,20 @@ __global__ __launch_bounds__(LB_THREADS) void layout_build_kernel(
 //   meta[g] = (first slot of part 0, first partial-tile slot or -1, ordinal among split groups or -1, parts)
 
 struct GroupPlan {
-    int parts;      // workgroup-sized pieces the group is cut into
+    int parts;      // workgroup-sized pieces the group is cut into (or row slices, see below)
     int len;
+    bool sliced;    // the whole group goes to SCHED_ROW_SLICES waves, each taking some of its 32 element rows
 };
 
-__device__ __forceinline__ GroupPlan plan_group(int len, int cap, int waves, int allow_split)
+__device__ __forceinline__ GroupPlan plan_group(int len, int cap, int waves, int allow_split, int slice_max)
 {
     GroupPlan p;
     p.len = len;
+    p.sliced = len <= slice_max;
+    if (p.sliced) {
+        p.parts = SCHED_ROW_SLICES;
+        return p;
+    }
     const int span = cap * waves;                       // pairs one workgroup takes at the target chunk size
     int parts = allow_split ? (len + span - 1) / span : 1;
     parts = parts < 1 ? 1 : (parts > SCHED_MAX_PARTS ? SCHED_MAX_PARTS : parts);
@@ -118,30 +124,41 @@ __device__ __forceinline__ int waves_of_part(int part_len, int cap, int waves)
 }
 
 __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
-    const int *__restrict__ offsets, int groups, int cap, int waves, int allow_split,
+    const int *__restrict__ offsets, int groups, int cap, int waves, int allow_split, int slice_max,
     int4 *__restrict__ sched, int slot_capacity, int *__restrict__ counts_out)
 {
     __shared__ int total_slots;
     const int tid = (int)threadIdx.x;
     int4 *meta = sched;
     int4 *slots = sched + groups;
-    // serial first-fit: a team (the waves of one part) never straddles a workgroup boundary
+    // Serial first-fit.  Row-sliced groups come first and fill whole workgroups of their own (their
+    // waves need no barrier); then the others: a team (the waves of one part) never straddles a
+    // workgroup boundary.
     if (tid == 0) {
         int pos = 0, tile_slots = 0, split_groups = 0;
-        for (int g = 0; g < groups; ++g) {
-            const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split);
-            int first = -1;
-            for (int p = 0; p < gp.parts; ++p) {
-                int plen = piece_lo(gp.len, p + 1, gp.parts) - piece_lo(gp.len, p, gp.parts);
-                int nw = waves_of_part(plen, cap, waves);
-                int in_wg = pos % waves;
-                if (in_wg + nw > waves) pos += waves - in_wg;
-                if (p == 0) first = pos;
-                pos += nw;
+        for (int pass = 0; pass < 2; ++pass) {
+            for (int g = 0; g < groups; ++g) {
+                const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split, slice_max);
+                if (gp.sliced != (pass == 0)) continue;
+                if (gp.sliced) {
+                    meta[g] = make_int4(pos, -1, -1, gp.parts);
+                    pos += gp.parts;
+                    continue;
+                }
+                int first = -1;
+                for (int p = 0; p < gp.parts; ++p) {
+                    int plen = piece_lo(gp.len, p + 1, gp.parts) - piece_lo(gp.len, p, gp.parts);
+                    int nw = waves_of_part(plen, cap, waves);
+                    int in_wg = pos % waves;
+                    if (in_wg + nw > waves) pos += waves - in_wg;
+                    if (p == 0) first = pos;
+                    pos += nw;
+                }
+                const bool split = gp.parts > 1;
+                meta[g] = make_int4(first, split ? tile_slots : -1, split ? split_groups : -1, gp.parts);
+                if (split) { tile_slots += gp.parts; split_groups += 1; }
             }
-            const bool split = gp.parts > 1;
-            meta[g] = make_int4(first, split ? tile_slots : -1, split ? split_groups : -1, gp.parts);
-            if (split) { tile_slots += gp.parts; split_groups += 1; }
+            if (pass == 0) pos = (pos + waves - 1) / waves * waves;
         }
         int n_wgs = (pos + waves - 1) / waves;
         total_slots = n_wgs * waves;
@@ -156,8 +173,14 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
     __syncthreads();
     for (int g = tid; g < groups; g += LB_THREADS) {
         const int lo = offsets[g];
-        const GroupPlan gp = plan_group(offsets[g + 1] - lo, cap, waves, allow_split);
+        const GroupPlan gp = plan_group(offsets[g + 1] - lo, cap, waves, allow_split, slice_max);
         int pos = meta[g].x;
+        if (gp.sliced) {
+            for (int t = 0; t < gp.parts; ++t)
+                if (pos + t < slot_capacity)
+                    slots[pos + t] = make_int4(g, lo, lo + gp.len, sched_team_word((pos + t) % waves, 1, t, gp.parts));
+            continue;
+        }
         for (int p = 0; p < gp.parts; ++p) {
             const int pb = piece_lo(gp.len, p, gp.parts), pe = piece_lo(gp.len, p + 1, gp.parts);
             const int plen = pe - pb;
@@ -187,10 +210,10 @@ hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_b
 }
 
 hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                                 int allow_split, int32_t *sched, int64_t capacity,
+                                 int allow_split, int slice_max, int32_t *sched, int64_t capacity,
                                  int32_t *counts_out, hipStream_t stream)
 {
-    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, allow_split,
+    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, allow_split, slice_max,
                                                        (int4 *)sched, (int)(capacity - groups),
                                                        counts_out);
     return hipGetLastError();

@@ -56,7 +56,10 @@ __device__ int g_ablate = 0;   // 1: no LDS/MFMA, 2: no dense loads, 4: no spars
 #endif
 
 constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + 4 KB), reused for the fp32 partial tile
-constexpr int GW_PREFETCH_DEPTH = 2;    // pairs whose operands are in flight per wave: deeper costs 24 VGPRs a
+#ifndef BSA_GW_DEPTH
+#define BSA_GW_DEPTH 2
+#endif
+constexpr int GW_PREFETCH_DEPTH = BSA_GW_DEPTH;    // pairs whose operands are in flight per wave: deeper costs 24 VGPRs a
                                         // stage and did not pay (124 VGPRs = 4 waves per SIMD at depth 2)
 constexpr int SDD_KB_MAX = 4;           // k-blocks (of 32) whose operands stay resident per wave
 constexpr int SDD_LDS_PER_WAVE = 2048 * (1 + SDD_KB_MAX);   // a / result tile + one b tile per k-block

@@ -24,6 +24,13 @@
 
 namespace bsa {
 
+#ifdef BSA_TRACE
+__device__ int g_sm_ablate = 0;   // debug builds: 8 = no stores, 16 = no loads
+#define SM_ABLATE(bit) (g_sm_ablate & (bit))
+#else
+#define SM_ABLATE(bit) 0
+#endif
+
 constexpr int SM_MAX_WAVES = 8;
 
 template <typename T> struct Chunk;
@@ -83,10 +90,181 @@ struct AddOp { __device__ __forceinline__ float operator()(float a, float b) con
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// scaled scores of one 16-byte chunk that starts at (row, col0) of block column bcol of block row
+// `group`; with `causal`, columns right of the diagonal count as -inf
+template <typename T>
+__device__ __forceinline__ void scaled_chunk(const uint4 &raw, int row, int col0, int bcol, int group,
+                                             float scale2, int causal, float (&v)[Chunk<T>::EPC])
+{
+    constexpr int EPC = Chunk<T>::EPC;
+    Chunk<T>::unpack(raw, v);
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) v[i] *= scale2;
+    if (causal && bcol >= group) {
+        const int limit = (bcol > group) ? -1 : row;   // last visible column inside the block
+#pragma unroll
+        for (int i = 0; i < EPC; ++i)
+            if (col0 + i > limit) v[i] = -__builtin_inff();
+    }
+}
+
+// Hides a register from common-subexpression elimination: the second pass over a register-resident
+// slice must RE-derive the scaled scores from the packed data, not keep every unpacked float of the
+// first pass alive (that is 2-4x the registers of the slice itself).
+__device__ __forceinline__ void launder(uint4 &r)
+{
+    asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
+}
+
+__device__ __forceinline__ float finite_or_zero(float m) { return m == -__builtin_inff() ? 0.f : m; }
+
+// ---------------------------------------------------------------------------
+// Row-sliced walk: a block row of at most CBS blocks goes whole to two wavefronts,
+// each owning 16 of the 32 element rows.  The wave issues every load of its slice
+// at once (one 16-byte request per lane and block for fp16), keeps the slice in
+// registers, and needs neither LDS nor a barrier: a row lives in LPR neighbouring
+// lanes.  NS = 16-byte chunks per lane and block of a slice.
+// ---------------------------------------------------------------------------
+template <typename T, int CBS>
+__device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *__restrict__ yb,
+                                                   const BlockDesc *__restrict__ blocks, const SchedEntry &e,
+                                                   float scale2, int causal)
+{
+    typedef Chunk<T> C;
+    constexpr int NS = C::NQ / SCHED_ROW_SLICES, EPC = C::EPC, LPR = C::LPR;
+    constexpr int ROWS_PER_Q = WAVE / LPR;
+    const int l = lane_id();
+    const int n = e.end - e.begin;
+    const int row_base = (BS / SCHED_ROW_SLICES) * e.part() + l / LPR;   // + q * ROWS_PER_Q
+    const int col0 = EPC * (l % LPR);
+    const int slice_off = (BS2 / SCHED_ROW_SLICES) * e.part() + l * EPC;  // + q * 64 * EPC, inside a block
+    const float NEG_INF = -__builtin_inff();
+
+    float m[NS], s[NS];
+#pragma unroll
+    for (int q = 0; q < NS; ++q) { m[q] = NEG_INF; s[q] = 0.f; }
+    DescWindow win;
+    win.fetch(blocks, e.begin, e.end);
+
+    if (n <= CBS) {
+        // block indices and columns are re-read from the window (v_readlane) in every pass:
+        // keeping 2 x CBS scalars alive would spill
+        uint4 raw[CBS][NS];
+#pragma unroll
+        for (int j = 0; j < CBS; ++j) {
+            if (j < n) {
+                const BlockDesc d = win.get(e.begin + j);
+#pragma unroll
+                for (int q = 0; q < NS; ++q)
+                    raw[j][q] = SM_ABLATE(16) ? make_uint4(d.idx, j, q, l)
+                                              : ldg16(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CBS; ++j) {
+            if (j < n) {
+#pragma unroll
+                for (int q = 0; q < NS; ++q) {
+                    float v[EPC];
+                    scaled_chunk<T>(raw[j][q], row_base + q * ROWS_PER_Q, col0, win.get(e.begin + j).col(), e.group, scale2,
+                                    causal, v);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) m[q] = fmaxf(m[q], v[i]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);   // one block at a time: unpacking them all at once spills
+        }
+#pragma unroll
+        for (int q = 0; q < NS; ++q) m[q] = finite_or_zero(row_allreduce<LPR>(m[q], MaxOp()));
+#pragma unroll
+        for (int j = 0; j < CBS; ++j) {
+            if (j < n) {
+#pragma unroll
+                for (int q = 0; q < NS; ++q) {
+                    float v[EPC];
+                    launder(raw[j][q]);
+                    scaled_chunk<T>(raw[j][q], row_base + q * ROWS_PER_Q, col0, win.get(e.begin + j).col(), e.group, scale2,
+                                    causal, v);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) {
+                        v[i] = exp2_fast(v[i] - m[q]);
+                        s[q] += v[i];
+                    }
+                    raw[j][q] = C::pack(v);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+            s[q] = row_allreduce<LPR>(s[q], AddOp());
+            s[q] = s[q] > 0.f ? 1.f / s[q] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < CBS; ++j) {
+            if (j < n) {
+#pragma unroll
+                for (int q = 0; q < NS; ++q) {
+                    float v[EPC];
+                    C::unpack(raw[j][q], v);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) v[i] *= s[q];
+                    if (!SM_ABLATE(8) || v[0] == 1234.5f)
+                        stg16(yb + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
+    }
+
+    // longer than the register capacity (a schedule built with another slice_max): two passes
+    for (int p = e.begin; p < e.end; ++p) {
+        if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+        const BlockDesc d = win.get(p);
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+            float v[EPC];
+            scaled_chunk<T>(ldg16(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
+                            row_base + q * ROWS_PER_Q, col0, d.col(), e.group, scale2, causal, v);
+            float bm = v[0];
+#pragma unroll
+            for (int i = 1; i < EPC; ++i) bm = fmaxf(bm, v[i]);
+            const float nm = fmaxf(m[q], bm);
+            const float mm = finite_or_zero(nm);
+            float acc = s[q] * exp2_fast(m[q] - mm);
+#pragma unroll
+            for (int i = 0; i < EPC; ++i) acc += exp2_fast(v[i] - mm);
+            s[q] = acc;
+            m[q] = nm;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NS; ++q) {
+        const float rm = finite_or_zero(row_allreduce<LPR>(m[q], MaxOp()));
+        s[q] = row_allreduce<LPR>(s[q] * exp2_fast(m[q] - rm), AddOp());
+        s[q] = s[q] > 0.f ? 1.f / s[q] : 0.f;
+        m[q] = rm;
+    }
+    for (int p = e.begin; p < e.end; ++p) {
+        if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+        const BlockDesc d = win.get(p);
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+            float v[EPC];
+            scaled_chunk<T>(ldg16(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
+                            row_base + q * ROWS_PER_Q, col0, d.col(), e.group, scale2, causal, v);
+#pragma unroll
+            for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - m[q]) * s[q];
+            stg16(yb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------
-template <typename T, int CB>
+template <typename T, int CB, int CBS>
 __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
     const T *__restrict__ x, T *__restrict__ y, const BlockDesc *__restrict__ blocks,
     const SchedEntry *__restrict__ sched, int n_swg, int batches, int nnz,
@@ -106,22 +284,18 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
     const int n = active ? e.end - e.begin : 0;
     const T *xb = x + (size_t)batch * nnz * BS2;
     T *yb = y + (size_t)batch * nnz * BS2;
+
+    // Row-sliced waves fill workgroups of their own (the schedule builder sees to that), so this
+    // branch is uniform over the workgroup and the barrier below is never left waiting.
+    if (active && e.parts() > 1) {
+        softmax_fwd_sliced<T, CBS>(xb, yb, blocks, e, scale2, causal);
+        return;
+    }
+    if (sched[swg * W].parts() > 1) return;   // an unused slot behind the last row-sliced waves
+
     const int col0 = EPC * (l % LPR);          // first column of this lane's chunk inside a block
     const int row0 = l / LPR;                  // element row of chunk q is row0 + q * ROWS_PER_Q
     const float NEG_INF = -__builtin_inff();
-
-    // scaled scores of one chunk, masked
-    auto scaled = [&](const uint4 &raw, int q, int bcol, float (&v)[EPC]) {
-        C::unpack(raw, v);
-#pragma unroll
-        for (int i = 0; i < EPC; ++i) v[i] *= scale2;
-        if (causal && bcol >= e.group) {
-            int limit = (bcol > e.group) ? -1 : row0 + q * ROWS_PER_Q;   // last visible column in the block
-#pragma unroll
-            for (int i = 0; i < EPC; ++i)
-                if (col0 + i > limit) v[i] = NEG_INF;
-        }
-    };
 
     float m[NQ], s[NQ];
 #pragma unroll
@@ -151,7 +325,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     float v[EPC];
-                    scaled(raw[j][q], q, bcol[j], v);
+                    scaled_chunk<T>(raw[j][q], row0 + q * ROWS_PER_Q, col0, bcol[j], e.group, scale2, causal, v);
 #pragma unroll
                     for (int i = 0; i < EPC; ++i) m[q] = fmaxf(m[q], v[i]);
                 }
@@ -166,8 +340,9 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     float v[EPC];
-                    scaled(raw[j][q], q, bcol[j], v);
-                    const float mm = (m[q] == NEG_INF) ? 0.f : m[q];
+                    launder(raw[j][q]);
+                    scaled_chunk<T>(raw[j][q], row0 + q * ROWS_PER_Q, col0, bcol[j], e.group, scale2, causal, v);
+                    const float mm = finite_or_zero(m[q]);
 #pragma unroll
                     for (int i = 0; i < EPC; ++i) {
                         v[i] = exp2_fast(v[i] - mm);
@@ -186,12 +361,13 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
                 float v[EPC];
-                scaled(ldg16(src + (l + WAVE * q) * EPC), q, d.col(), v);
+                scaled_chunk<T>(ldg16(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
+                                scale2, causal, v);
                 float bm = v[0];
 #pragma unroll
                 for (int i = 1; i < EPC; ++i) bm = fmaxf(bm, v[i]);
                 const float nm = fmaxf(m[q], bm);
-                const float mm = (nm == NEG_INF) ? 0.f : nm;
+                const float mm = finite_or_zero(nm);
                 float acc = s[q] * exp2_fast(m[q] - mm);
 #pragma unroll
                 for (int i = 0; i < EPC; ++i) acc += exp2_fast(v[i] - mm);
@@ -203,8 +379,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
             const float rm = row_allreduce<LPR>(m[q], MaxOp());
-            const float mm = (rm == NEG_INF) ? 0.f : rm;
-            s[q] *= exp2_fast(m[q] - mm);
+            s[q] *= exp2_fast(m[q] - finite_or_zero(rm));
             m[q] = rm;
         }
     }
@@ -227,19 +402,18 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
         if (nw > 1) {
             M = NEG_INF;
             for (int t = 0; t < nw; ++t) M = fmaxf(M, stats[slot0 + t][row0 + q * ROWS_PER_Q].x);
-            const float MM = (M == NEG_INF) ? 0.f : M;
+            const float MM = finite_or_zero(M);
             S = 0.f;
             for (int t = 0; t < nw; ++t) {
                 const float2 st = stats[slot0 + t][row0 + q * ROWS_PER_Q];
                 S += st.y * exp2_fast(st.x - MM);
             }
         }
-        const float MM = (M == NEG_INF) ? 0.f : M;
+        const float MM = finite_or_zero(M);
         const float inv = S > 0.f ? 1.f / S : 0.f;
         gm[q] = MM;
         inv_s[q] = inv;
-        f[q] = exp2_fast(((m[q] == NEG_INF) ? 0.f : m[q]) - MM) * inv;
-        if (m[q] == NEG_INF) f[q] = 0.f;
+        f[q] = (m[q] == NEG_INF) ? 0.f : exp2_fast(m[q] - MM) * inv;
     }
 
     if (resident) {
@@ -267,7 +441,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
                 float v[EPC];
-                scaled(ldg16(src + (l + WAVE * q) * EPC), q, d.col(), v);
+                scaled_chunk<T>(ldg16(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
+                                scale2, causal, v);
 #pragma unroll
                 for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - gm[q]) * inv_s[q];
                 stg16(dst + (l + WAVE * q) * EPC, C::pack(v));
@@ -279,7 +454,85 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 // ---------------------------------------------------------------------------
 // backward: dx = scale * (dy - sum_row(dy * y)) * y
 // ---------------------------------------------------------------------------
-template <typename T, int CB>
+template <typename T, int CBS>
+__device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, const T *__restrict__ dy,
+                                                   T *__restrict__ dx, const BlockDesc *__restrict__ blocks,
+                                                   const SchedEntry &e, float scale)
+{
+    typedef Chunk<T> C;
+    constexpr int NS = C::NQ / SCHED_ROW_SLICES, EPC = C::EPC, LPR = C::LPR;
+    const int l = lane_id();
+    const int n = e.end - e.begin;
+    const int slice_off = (BS2 / SCHED_ROW_SLICES) * e.part() + l * EPC;
+    float dot[NS];
+#pragma unroll
+    for (int q = 0; q < NS; ++q) dot[q] = 0.f;
+    DescWindow win;
+    win.fetch(blocks, e.begin, e.end);
+
+    auto finish = [&](const uint4 &uy, const uint4 &ud, int q) {
+        float a[EPC], b[EPC];
+        C::unpack(uy, a);
+        C::unpack(ud, b);
+#pragma unroll
+        for (int i = 0; i < EPC; ++i) a[i] = scale * (b[i] - dot[q]) * a[i];
+        return C::pack(a);
+    };
+    auto accumulate = [&](const uint4 &uy, const uint4 &ud, int q) {
+        float a[EPC], b[EPC];
+        C::unpack(uy, a);
+        C::unpack(ud, b);
+#pragma unroll
+        for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
+    };
+
+    if (n <= CBS) {
+        uint4 ry[CBS][NS], rd[CBS][NS];
+#pragma unroll
+        for (int j = 0; j < CBS; ++j) {
+            if (j < n) {
+                const size_t o = (size_t)win.get(e.begin + j).idx * BS2 + slice_off;
+#pragma unroll
+                for (int q = 0; q < NS; ++q) {
+                    ry[j][q] = ldg16(y + o + q * WAVE * EPC);
+                    rd[j][q] = ldg16(dy + o + q * WAVE * EPC);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CBS; ++j)
+            if (j < n)
+#pragma unroll
+                for (int q = 0; q < NS; ++q) accumulate(ry[j][q], rd[j][q], q);
+#pragma unroll
+        for (int q = 0; q < NS; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
+#pragma unroll
+        for (int j = 0; j < CBS; ++j)
+            if (j < n)
+#pragma unroll
+                for (int q = 0; q < NS; ++q)
+                    stg16(dx + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC,
+                          finish(ry[j][q], rd[j][q], q));
+        return;
+    }
+    for (int p = e.begin; p < e.end; ++p) {
+        if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+        const size_t o = (size_t)win.get(p).idx * BS2 + slice_off;
+#pragma unroll
+        for (int q = 0; q < NS; ++q) accumulate(ldg16(y + o + q * WAVE * EPC), ldg16(dy + o + q * WAVE * EPC), q);
+    }
+#pragma unroll
+    for (int q = 0; q < NS; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
+    for (int p = e.begin; p < e.end; ++p) {
+        if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+        const size_t o = (size_t)win.get(p).idx * BS2 + slice_off;
+#pragma unroll
+        for (int q = 0; q < NS; ++q)
+            stg16(dx + o + q * WAVE * EPC, finish(ldg16(y + o + q * WAVE * EPC), ldg16(dy + o + q * WAVE * EPC), q));
+    }
+}
+
+template <typename T, int CB, int CBS>
 __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
     const T *__restrict__ y, const T *__restrict__ dy, T *__restrict__ dx,
     const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
@@ -299,6 +552,12 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
     const int n = active ? e.end - e.begin : 0;
     const size_t boff = (size_t)batch * nnz * BS2;
     const int row0 = l / LPR;
+
+    if (active && e.parts() > 1) {   // row-sliced waves sit in workgroups of their own
+        softmax_bwd_sliced<T, CBS>(y + boff, dy + boff, dx + boff, blocks, e, scale);
+        return;
+    }
+    if (sched[swg * W].parts() > 1) return;
 
     float dot[NQ];
 #pragma unroll
@@ -407,11 +666,11 @@ hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t s
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
     const float scale2 = p.scale * 1.4426950408889634f;
     if (dtype == BSA_F16)
-        softmax_fwd_kernel<half_t, 8><<<grid, block, 0, st>>>(
+        softmax_fwd_kernel<half_t, 4, 24><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (half_t *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
     else
-        softmax_fwd_kernel<float, 4><<<grid, block, 0, st>>>(
+        softmax_fwd_kernel<float, 2, 12><<<grid, block, 0, st>>>(
             (const float *)p.x, (float *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
     return hipGetLastError();
@@ -421,14 +680,23 @@ hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t 
 {
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
     if (dtype == BSA_F16)
-        softmax_bwd_kernel<half_t, 4><<<grid, block, 0, st>>>(
+        softmax_bwd_kernel<half_t, 2, 12><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (const half_t *)p.dy, (half_t *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     else
-        softmax_bwd_kernel<float, 2><<<grid, block, 0, st>>>(
+        softmax_bwd_kernel<float, 1, 6><<<grid, block, 0, st>>>(
             (const float *)p.x, (const float *)p.dy, (float *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     return hipGetLastError();
 }
+
+#ifdef BSA_TRACE
+}  // namespace bsa
+extern "C" int bsa_debug_sm_ablate(int bits)
+{
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(bsa::g_sm_ablate), &bits, sizeof(bits));
+}
+namespace bsa {
+#endif
 
 }  // namespace bsa

@@ -14,6 +14,9 @@ BLOCK = 32
 SCHEDULE_GROUP_WALK = (12, 2)
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
+# block rows of at most this many blocks are handed whole to two wavefronts (16 element rows each),
+# which keep them in registers and need no exchange; per dtype: forward, backward
+SOFTMAX_SLICE_MAX = {torch.float16: (24, 12), torch.float32: (12, 6)}
 
 _DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
 
@@ -21,13 +24,14 @@ _DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
 class Schedule:
     """Device-resident wavefront schedule of one offset table."""
 
-    def __init__(self, offsets: torch.Tensor, nnz: int, cap: int, waves: int, allow_split: bool = True):
+    def __init__(self, offsets: torch.Tensor, nnz: int, cap: int, waves: int, allow_split: bool = True,
+                 slice_max: int = -1):
         groups = offsets.numel() - 1
         capacity = _k.lib.bsa_schedule_capacity(groups, nnz, cap, waves)
         self.table = torch.empty(4 * capacity, dtype=torch.int32, device=offsets.device)
         counts = torch.empty(4, dtype=torch.int32, device=offsets.device)
         with torch.cuda.device(offsets.device):
-            _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves, int(allow_split),
+            _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves, int(allow_split), slice_max,
                                                self.table.data_ptr(), capacity, counts.data_ptr(),
                                                _k.current_stream()))
         self.workgroups, self.tile_slots, self.split_groups, self.slots = (int(v) for v in counts.tolist())
@@ -63,9 +67,9 @@ def schedule_for(layout, kind):
     return cache[kind]
 
 
-def _softmax_schedule(layout):
+def _softmax_schedule(layout, dtype, backward):
     cap, waves = SCHEDULE_SOFTMAX
-    return schedule_for(layout, (cap, waves, False))
+    return schedule_for(layout, (cap, waves, False, SOFTMAX_SLICE_MAX[dtype][1 if backward else 0]))
 
 
 def _check_layout(layout, name):
@@ -171,7 +175,7 @@ def sparse_softmax_forward(x, row_blocks, row_table, scale=1.0, causal=False, co
     y = torch.empty_like(x)
     if nnz == 0 or x.numel() == 0:
         return y
-    sched = _softmax_schedule(row_layout)
+    sched = _softmax_schedule(row_layout, x.dtype, False)
     with torch.cuda.device(x.device):
         _k.check(_k.lib.bsa_softmax_forward(
             _DTYPES[x.dtype], x.data_ptr(), y.data_ptr(), row_blocks.data_ptr(), row_table.data_ptr(),
@@ -191,7 +195,7 @@ def sparse_softmax_backward(y, dy, row_blocks, row_table, scale=1.0, col_layout=
     dx = torch.empty_like(y)
     if nnz == 0 or y.numel() == 0:
         return dx
-    sched = _softmax_schedule(row_layout)
+    sched = _softmax_schedule(row_layout, y.dtype, True)
     with torch.cuda.device(y.device):
         _k.check(_k.lib.bsa_softmax_backward(
             _DTYPES[y.dtype], y.data_ptr(), dy.data_ptr(), dx.data_ptr(), row_blocks.data_ptr(),

@@ -86,6 +86,11 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
  * most that many pairs when `allow_split` != 0 (matmul), and gets longer
  * chunks otherwise (softmax, whose rows cannot be split across workgroups).
  * Empty groups get one wavefront with an empty chunk (it writes the zeros).
+ * With `slice_max` >= 0 (softmax only) a group of at most slice_max pairs is not
+ * chunked at all: it goes whole to two wavefronts, each taking 16 of its 32
+ * element rows (team word: waves = 1, part = slice, parts = 2), and these
+ * wavefronts fill workgroups of their own at the front of the schedule.  Pass
+ * -1 for the matmul schedules.
  * No counterpart in the reference, whose grids are (nnz, B) and
  * (B, M/32, N/32) (sparse/native/sparse_smm_gpu.cu:278-279).
  *   sched        device int32[4 * bsa_schedule_capacity(...)]
@@ -94,7 +99,7 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
  */
 int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves);
 int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                       int allow_split, int32_t *sched, int64_t capacity,
+                       int allow_split, int slice_max, int32_t *sched, int64_t capacity,
                        int32_t *counts_out, void *stream);
 
 /* ---- block-sparse matmul -----------------------------------------------
