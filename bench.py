@@ -154,9 +154,20 @@ def main():
             per_op[name]["nnz_TFLOPs"] = round(tf, 2)
             per_op[name]["mfma_frac"] = round(tf / MFMA_F16_PEAK_TFLOPS, 4)
 
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/): same
+    # workload, same kernels; absent file -> null
+    traffic = {}
+    try:
+        with open(os.path.join(ROOT, "profiles", "bench_seq4096_hbm_traffic.json")) as f:
+            traffic = json.load(f)["traffic"]
+    except (OSError, ValueError, KeyError):
+        pass
+    for name in per_op:
+        per_op[name]["traffic_bytes"] = traffic.get(name)
+
     dominant = max(("sdd", "dsd", "dds"), key=lambda n: per_op[n]["us"])
     roofline = {"kernel": dominant, "bound": "hbm", "achieved": per_op[dominant]["GBps"], "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": per_op[dominant]["hbm_frac"], "traffic": None}
+                "unit": "GB/s", "frac": per_op[dominant]["hbm_frac"], "traffic": traffic.get(dominant)}
 
     result = {
         "metric": "nnz-block TFLOP/s SDD/DSD/DDS fp16 @seq4096; softmax GB/s; % of roofline",
@@ -168,7 +179,8 @@ def main():
         "roofline": roofline,
         "softmax": {"GBps": per_op["softmax"]["GBps"], "us": per_op["softmax"]["us"],
                     "roofline": {"bound": "hbm", "achieved": per_op["softmax"]["GBps"], "peak": HBM_PEAK_GBS,
-                                 "unit": "GB/s", "frac": per_op["softmax"]["hbm_frac"], "traffic": None}},
+                                 "unit": "GB/s", "frac": per_op["softmax"]["hbm_frac"],
+                                 "traffic": traffic.get("softmax")}},
         "kernels": per_op,
     }
 
