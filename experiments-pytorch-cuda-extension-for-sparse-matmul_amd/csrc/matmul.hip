@@ -44,11 +44,15 @@ __device__ __forceinline__ void trace_wave(const unsigned long long (&t)[5], int
 #define BSA_TRACE_MARK(i) { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); trace_t[i] = wall_clock64(); }
 #define BSA_TRACE_MARK_NOWAIT(i) { trace_t[i] = wall_clock64(); }
 __device__ int g_ablate = 0;   // 1: no LDS/MFMA, 2: no dense loads, 4: no sparse loads
-#define BSA_ABLATE(bit) (g_ablate & (bit))
-#define BSA_TRACE_BEGIN unsigned long long trace_t[5]; trace_t[0] = trace_t[1] = trace_t[2] = trace_t[3] = trace_t[4] = wall_clock64();
+#define BSA_ABLATE(bit) (ablate_bits & (bit))
+#define BSA_TRACE_BEGIN const int ablate_bits = __builtin_amdgcn_readfirstlane(g_ablate); unsigned long long trace_t[5]; trace_t[0] = trace_t[1] = trace_t[2] = trace_t[3] = trace_t[4] = wall_clock64();
 #define BSA_TRACE_END(batch, group, n) trace_wave(trace_t, batch, group, n);
 #else
+#ifdef BSA_ABLATE_BITS
+#define BSA_ABLATE(bit) ((BSA_ABLATE_BITS) & (bit))
+#else
 #define BSA_ABLATE(bit) 0
+#endif
 #define BSA_TRACE_MARK(i)
 #define BSA_TRACE_MARK_NOWAIT(i)
 #define BSA_TRACE_BEGIN
@@ -364,9 +368,11 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     BSA_TRACE_BEGIN
     int batch, swg;
     if (!map_workgroup(n_swg, batches, batch, swg)) return;   // whole workgroup leaves together
+    if (BSA_ABLATE(32)) return;
     const int w = wave_id(), l = lane_id();
     const int W = (int)(blockDim.x >> 6);
     const SchedEntry e = sched[swg * W + w];
+    if (BSA_ABLATE(64)) { if (e.group == 12345678) out[0] = (half_t)1; return; }
     const int y0 = 64 * (int)blockIdx.y;
     const int ytiles = (DN - y0) >= 64 ? 2 : 1;
 
@@ -442,6 +448,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
         for (int seg = e.begin; seg < e.end; seg += WAVE) {
             const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
             win.fetch(blocks, seg, seg_end);
+            if (BSA_ABLATE(128)) { if (win.idx == 12345678) out[0] = (half_t)1; return; }
 #pragma unroll
             for (int d = 0; d < DEPTH; ++d)
                 if (seg + d < seg_end) load(seg + d, fr[d]);
@@ -459,6 +466,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     }
 
     BSA_TRACE_MARK(3)
+    if (BSA_ABLATE(256)) { if (acc[0][0] == 1234.5f) out[0] = (half_t)1; return; }
     const bool store_it = team_reduce(acc, e, w, lds_raw) &&
                           (e.parts() <= 1 || split_combine(acc, e, sched_groups[e.group], ws, batch));
     BSA_TRACE_MARK(4)
