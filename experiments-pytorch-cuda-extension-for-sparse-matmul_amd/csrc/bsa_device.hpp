@@ -142,6 +142,20 @@ __device__ __forceinline__ f16v mfma_f32(float a, float b, f16v c)
 __device__ __forceinline__ uint4 ldg16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
 __device__ __forceinline__ void stg16(void *p, uint4 v) { *reinterpret_cast<uint4 *>(p) = v; }
 
+// Streaming variants for data that is touched once (sparse blocks, softmax scores, block results):
+// the nt hint keeps it from displacing the dense operand tiles that are re-read out of L2.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ldg16_stream(const void *p)
+{
+    u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stg16_stream(void *p, uint4 v)
+{
+    u32x4 w = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(p));
+}
+
 __device__ __forceinline__ h8 as_h8(uint4 v) { return __builtin_bit_cast(h8, v); }
 
 // 16 fp32 accumulators -> 16 halves in two 16-byte registers.

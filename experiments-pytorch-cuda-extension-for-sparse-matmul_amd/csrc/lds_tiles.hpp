@@ -111,12 +111,20 @@ __device__ __forceinline__ void lds_get_linear(const half_t *tile, uint4 (&raw)[
         raw[q] = *reinterpret_cast<const uint4 *>(lds_bytes(tile) + get_linear_addr(l, q));
 }
 
-// coalesced store of a 2 KB block
+// coalesced store of a 2 KB block (written once, not read again by this kernel)
 __device__ __forceinline__ void stg_tile32(half_t *dst, const uint4 (&raw)[2])
 {
     int l = lane_id();
-    stg16(dst + 8 * l, raw[0]);
-    stg16(dst + 8 * (l + 64), raw[1]);
+    stg16_stream(dst + 8 * l, raw[0]);
+    stg16_stream(dst + 8 * (l + 64), raw[1]);
+}
+
+// coalesced load of a contiguous 2 KB block that is read once
+__device__ __forceinline__ void ldg_block32_stream(const half_t *src, uint4 (&raw)[2])
+{
+    int l = lane_id();
+    raw[0] = ldg16_stream(src + 8 * l);
+    raw[1] = ldg16_stream(src + 8 * (l + 64));
 }
 
 }  // namespace bsa

@@ -389,7 +389,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     auto load = [&](int p, Frag &f) {
         const BlockDesc d = win.get(p);
         const int kblk = S_KC ? d.col() : d.row();
-        if (!BSA_ABLATE(4)) ldg_tile32(spb + (size_t)d.idx * BS2, BS, f.s);
+        if (!BSA_ABLATE(4)) ldg_block32_stream(spb + (size_t)d.idx * BS2, f.s);
         if (BSA_ABLATE(2)) return;
         if (D_KC) {          // stored [DN][KT]: two 32 x 32 tiles, rows KT apart
             const half_t *src = dnb + (size_t)y0 * KT + BS * kblk;

@@ -157,7 +157,7 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
 #pragma unroll
                 for (int q = 0; q < NS; ++q)
                     raw[j][q] = SM_ABLATE(16) ? make_uint4(d.idx, j, q, l)
-                                              : ldg16(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC);
+                                              : ldg16_stream(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC);
             }
         }
 #pragma unroll
@@ -210,7 +210,7 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
 #pragma unroll
                     for (int i = 0; i < EPC; ++i) v[i] *= s[q];
                     if (!SM_ABLATE(8) || v[0] == 1234.5f)
-                        stg16(yb + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
+                        stg16_stream(yb + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -225,7 +225,7 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
 #pragma unroll
         for (int q = 0; q < NS; ++q) {
             float v[EPC];
-            scaled_chunk<T>(ldg16(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
+            scaled_chunk<T>(ldg16_stream(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
                             row_base + q * ROWS_PER_Q, col0, d.col(), e.group, scale2, causal, v);
             float bm = v[0];
 #pragma unroll
@@ -252,11 +252,11 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
 #pragma unroll
         for (int q = 0; q < NS; ++q) {
             float v[EPC];
-            scaled_chunk<T>(ldg16(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
+            scaled_chunk<T>(ldg16_stream(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
                             row_base + q * ROWS_PER_Q, col0, d.col(), e.group, scale2, causal, v);
 #pragma unroll
             for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - m[q]) * s[q];
-            stg16(yb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
+            stg16_stream(yb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
         }
     }
 }
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
                 bidx[j] = d.idx; bcol[j] = d.col();
                 const T *src = xb + (size_t)d.idx * BS2;
 #pragma unroll
-                for (int q = 0; q < NQ; ++q) raw[j][q] = ldg16(src + (l + WAVE * q) * EPC);
+                for (int q = 0; q < NQ; ++q) raw[j][q] = ldg16_stream(src + (l + WAVE * q) * EPC);
             }
         }
         // pass 1 (registers): row max
@@ -361,7 +361,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
                 float v[EPC];
-                scaled_chunk<T>(ldg16(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
+                scaled_chunk<T>(ldg16_stream(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
                                 scale2, causal, v);
                 float bm = v[0];
 #pragma unroll
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
                     C::unpack(raw[j][q], v);
 #pragma unroll
                     for (int i = 0; i < EPC; ++i) v[i] *= f[q];
-                    stg16(dst + (l + WAVE * q) * EPC, C::pack(v));
+                    stg16_stream(dst + (l + WAVE * q) * EPC, C::pack(v));
                 }
             }
         }
@@ -441,11 +441,11 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
                 float v[EPC];
-                scaled_chunk<T>(ldg16(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
+                scaled_chunk<T>(ldg16_stream(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
                                 scale2, causal, v);
 #pragma unroll
                 for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - gm[q]) * inv_s[q];
-                stg16(dst + (l + WAVE * q) * EPC, C::pack(v));
+                stg16_stream(dst + (l + WAVE * q) * EPC, C::pack(v));
             }
         }
     }
@@ -494,8 +494,8 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
                 const size_t o = (size_t)win.get(e.begin + j).idx * BS2 + slice_off;
 #pragma unroll
                 for (int q = 0; q < NS; ++q) {
-                    ry[j][q] = ldg16(y + o + q * WAVE * EPC);
-                    rd[j][q] = ldg16(dy + o + q * WAVE * EPC);
+                    ry[j][q] = ldg16_stream(y + o + q * WAVE * EPC);
+                    rd[j][q] = ldg16_stream(dy + o + q * WAVE * EPC);
                 }
             }
         }
@@ -511,7 +511,7 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
             if (j < n)
 #pragma unroll
                 for (int q = 0; q < NS; ++q)
-                    stg16(dx + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC,
+                    stg16_stream(dx + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC,
                           finish(ry[j][q], rd[j][q], q));
         return;
     }
@@ -519,7 +519,7 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
         if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
         const size_t o = (size_t)win.get(p).idx * BS2 + slice_off;
 #pragma unroll
-        for (int q = 0; q < NS; ++q) accumulate(ldg16(y + o + q * WAVE * EPC), ldg16(dy + o + q * WAVE * EPC), q);
+        for (int q = 0; q < NS; ++q) accumulate(ldg16_stream(y + o + q * WAVE * EPC), ldg16_stream(dy + o + q * WAVE * EPC), q);
     }
 #pragma unroll
     for (int q = 0; q < NS; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
@@ -528,7 +528,7 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
         const size_t o = (size_t)win.get(p).idx * BS2 + slice_off;
 #pragma unroll
         for (int q = 0; q < NS; ++q)
-            stg16(dx + o + q * WAVE * EPC, finish(ldg16(y + o + q * WAVE * EPC), ldg16(dy + o + q * WAVE * EPC), q));
+            stg16_stream(dx + o + q * WAVE * EPC, finish(ldg16_stream(y + o + q * WAVE * EPC), ldg16_stream(dy + o + q * WAVE * EPC), q));
     }
 }
 
@@ -576,8 +576,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
                 const size_t o = boff + (size_t)bidx[j] * BS2;
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
-                    ry[j][q] = ldg16(y + o + (l + WAVE * q) * EPC);
-                    rd[j][q] = ldg16(dy + o + (l + WAVE * q) * EPC);
+                    ry[j][q] = ldg16_stream(y + o + (l + WAVE * q) * EPC);
+                    rd[j][q] = ldg16_stream(dy + o + (l + WAVE * q) * EPC);
                 }
             }
         }
@@ -601,8 +601,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
                 float a[EPC], b[EPC];
-                C::unpack(ldg16(y + o + (l + WAVE * q) * EPC), a);
-                C::unpack(ldg16(dy + o + (l + WAVE * q) * EPC), b);
+                C::unpack(ldg16_stream(y + o + (l + WAVE * q) * EPC), a);
+                C::unpack(ldg16_stream(dy + o + (l + WAVE * q) * EPC), b);
 #pragma unroll
                 for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
             }
@@ -641,7 +641,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
             if (j < n) {
                 const size_t o = boff + (size_t)bidx[j] * BS2;
 #pragma unroll
-                for (int q = 0; q < NQ; ++q) stg16(dx + o + (l + WAVE * q) * EPC, finish(ry[j][q], rd[j][q], q));
+                for (int q = 0; q < NQ; ++q) stg16_stream(dx + o + (l + WAVE * q) * EPC, finish(ry[j][q], rd[j][q], q));
             }
         }
     } else {
@@ -650,8 +650,8 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
             const size_t o = boff + (size_t)win.get(p).idx * BS2;
 #pragma unroll
             for (int q = 0; q < NQ; ++q)
-                stg16(dx + o + (l + WAVE * q) * EPC,
-                      finish(ldg16(y + o + (l + WAVE * q) * EPC), ldg16(dy + o + (l + WAVE * q) * EPC), q));
+                stg16_stream(dx + o + (l + WAVE * q) * EPC,
+                      finish(ldg16_stream(y + o + (l + WAVE * q) * EPC), ldg16_stream(dy + o + (l + WAVE * q) * EPC), q));
         }
     }
 }
