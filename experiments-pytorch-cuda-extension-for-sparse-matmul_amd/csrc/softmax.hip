@@ -51,6 +51,25 @@ template <> struct Chunk<half_t> {
         for (int i = 0; i < 8; ++i) h[i] = (half_t)v[i];
         return __builtin_bit_cast(uint4, h);
     }
+    // smallest and largest of the 8 halves, with packed fp16 min / max
+    static __device__ __forceinline__ void minmax(const uint4 &r, float &lo, float &hi)
+    {
+        const h2 a = __builtin_bit_cast(h2, r.x), b = __builtin_bit_cast(h2, r.y);
+        const h2 c = __builtin_bit_cast(h2, r.z), d = __builtin_bit_cast(h2, r.w);
+        const h2 mx = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+        const h2 mn = __builtin_elementwise_min(__builtin_elementwise_min(a, b), __builtin_elementwise_min(c, d));
+        hi = fmaxf((float)mx[0], (float)mx[1]);
+        lo = fminf((float)mn[0], (float)mn[1]);
+    }
+    // element i := `fill` where col0 + i > limit
+    static __device__ __forceinline__ void mask_right_of(uint4 &r, int col0, int limit, float fill)
+    {
+        h8 h = __builtin_bit_cast(h8, r);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (col0 + i > limit) h[i] = (half_t)fill;
+        r = __builtin_bit_cast(uint4, h);
+    }
 };
 template <> struct Chunk<float> {
     static constexpr int NQ = 4;
@@ -65,6 +84,22 @@ template <> struct Chunk<float> {
     {
         return make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]),
                           __float_as_uint(v[2]), __float_as_uint(v[3]));
+    }
+    static __device__ __forceinline__ void minmax(const uint4 &r, float &lo, float &hi)
+    {
+        float v[4];
+        unpack(r, v);
+        hi = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+        lo = fminf(fminf(v[0], v[1]), fminf(v[2], v[3]));
+    }
+    static __device__ __forceinline__ void mask_right_of(uint4 &r, int col0, int limit, float fill)
+    {
+        float v[4];
+        unpack(r, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (col0 + i > limit) v[i] = fill;
+        r = pack(v);
     }
 };
 
@@ -106,6 +141,40 @@ __device__ __forceinline__ void scaled_chunk(const uint4 &raw, int row, int col0
         for (int i = 0; i < EPC; ++i)
             if (col0 + i > limit) v[i] = -__builtin_inff();
     }
+}
+
+// Register-resident chunks: the causal mask is burnt into the packed data once (only blocks on or
+// right of the diagonal are touched, under a wave-uniform branch), the row max comes from packed
+// min / max of the raw scores, and the exponential is exp2(fma(x, scale2, -max)).
+template <typename T>
+__device__ __forceinline__ void mask_chunk(uint4 &raw, int row, int col0, int bcol, int group, float scale2)
+{
+    if (bcol >= group) {
+        const float fill = scale2 < 0.f ? __builtin_inff() : -__builtin_inff();   // -inf once scaled
+        Chunk<T>::mask_right_of(raw, col0, bcol > group ? -1 : row, fill);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ float chunk_scaled_max(const uint4 &raw, float scale2)
+{
+    float lo, hi;
+    Chunk<T>::minmax(raw, lo, hi);
+    return fmaxf(lo * scale2, hi * scale2);
+}
+
+// v[i] = exp2(scale2 * x[i] - m); returns their sum
+template <typename T>
+__device__ __forceinline__ float chunk_exp(const uint4 &raw, float scale2, float m, float (&v)[Chunk<T>::EPC])
+{
+    Chunk<T>::unpack(raw, v);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < Chunk<T>::EPC; ++i) {
+        v[i] = exp2_fast(__builtin_fmaf(v[i], scale2, -m));
+        sum += v[i];
+    }
+    return sum;
 }
 
 // Hides a register from common-subexpression elimination: the second pass over a register-resident
@@ -163,16 +232,13 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
 #pragma unroll
         for (int j = 0; j < CBS; ++j) {
             if (j < n) {
+                const int bcol = win.get(e.begin + j).col();
 #pragma unroll
                 for (int q = 0; q < NS; ++q) {
-                    float v[EPC];
-                    scaled_chunk<T>(raw[j][q], row_base + q * ROWS_PER_Q, col0, win.get(e.begin + j).col(), e.group, scale2,
-                                    causal, v);
-#pragma unroll
-                    for (int i = 0; i < EPC; ++i) m[q] = fmaxf(m[q], v[i]);
+                    if (causal) mask_chunk<T>(raw[j][q], row_base + q * ROWS_PER_Q, col0, bcol, e.group, scale2);
+                    m[q] = fmaxf(m[q], chunk_scaled_max<T>(raw[j][q], scale2));
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);   // one block at a time: unpacking them all at once spills
         }
 #pragma unroll
         for (int q = 0; q < NS; ++q) m[q] = finite_or_zero(row_allreduce<LPR>(m[q], MaxOp()));
@@ -182,18 +248,11 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
 #pragma unroll
                 for (int q = 0; q < NS; ++q) {
                     float v[EPC];
-                    launder(raw[j][q]);
-                    scaled_chunk<T>(raw[j][q], row_base + q * ROWS_PER_Q, col0, win.get(e.begin + j).col(), e.group, scale2,
-                                    causal, v);
-#pragma unroll
-                    for (int i = 0; i < EPC; ++i) {
-                        v[i] = exp2_fast(v[i] - m[q]);
-                        s[q] += v[i];
-                    }
+                    s[q] += chunk_exp<T>(raw[j][q], scale2, m[q], v);
                     raw[j][q] = C::pack(v);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_sched_barrier(0);   // one block at a time: unpacking them all at once spills
         }
 #pragma unroll
         for (int q = 0; q < NS; ++q) {
@@ -318,16 +377,14 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
                 for (int q = 0; q < NQ; ++q) raw[j][q] = ldg16_stream(src + (l + WAVE * q) * EPC);
             }
         }
-        // pass 1 (registers): row max
+        // pass 1 (registers): causal mask burnt in, row max
 #pragma unroll
         for (int j = 0; j < CB; ++j) {
             if (j < n) {
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
-                    float v[EPC];
-                    scaled_chunk<T>(raw[j][q], row0 + q * ROWS_PER_Q, col0, bcol[j], e.group, scale2, causal, v);
-#pragma unroll
-                    for (int i = 0; i < EPC; ++i) m[q] = fmaxf(m[q], v[i]);
+                    if (causal) mask_chunk<T>(raw[j][q], row0 + q * ROWS_PER_Q, col0, bcol[j], e.group, scale2);
+                    m[q] = fmaxf(m[q], chunk_scaled_max<T>(raw[j][q], scale2));
                 }
             }
         }
@@ -340,14 +397,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     float v[EPC];
-                    launder(raw[j][q]);
-                    scaled_chunk<T>(raw[j][q], row0 + q * ROWS_PER_Q, col0, bcol[j], e.group, scale2, causal, v);
-                    const float mm = finite_or_zero(m[q]);
-#pragma unroll
-                    for (int i = 0; i < EPC; ++i) {
-                        v[i] = exp2_fast(v[i] - mm);
-                        s[q] += v[i];
-                    }
+                    s[q] += chunk_exp<T>(raw[j][q], scale2, finite_or_zero(m[q]), v);
                     raw[j][q] = C::pack(v);
                 }
             }

@@ -11,7 +11,9 @@ from . import kernel as _k
 
 BLOCK = 32
 # tuning of the wavefront schedules: (target pairs per wavefront, wavefronts per workgroup)
-SCHEDULE_GROUP_WALK = (12, 2)
+SCHEDULE_GROUP_WALK = (12, 2)        # groups of at most GROUP_WALK_LONG pairs (rows of attention masks)
+SCHEDULE_GROUP_WALK_LONG = (8, 4)    # tables with longer groups (columns of causal / strided masks)
+GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
 # block rows of at most this many blocks are handed whole to two wavefronts (16 element rows each),
@@ -65,6 +67,20 @@ def schedule_for(layout, kind):
     if kind not in cache:
         cache[kind] = Schedule(offsets, blocks.numel() // 2, *kind)
     return cache[kind]
+
+
+def _longest_group(offsets) -> int:
+    """Pairs in the longest group of a table; measured once and kept on the offsets tensor."""
+    longest = getattr(offsets, "_bsa_longest", None)
+    if longest is None:
+        longest = int((offsets[1:] - offsets[:-1]).max().item()) if offsets.numel() > 1 else 0
+        offsets._bsa_longest = longest
+    return longest
+
+
+def _group_walk_schedule(layout):
+    kind = SCHEDULE_GROUP_WALK_LONG if _longest_group(layout[1]) > GROUP_WALK_LONG else SCHEDULE_GROUP_WALK
+    return schedule_for(layout, kind)
 
 
 def _softmax_schedule(layout, dtype, backward):
@@ -137,7 +153,7 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
         shape = batch_a + (num_blocks, BLOCK, BLOCK)
     c = torch.empty(shape, dtype=a.dtype, device=a.device)
 
-    sched = schedule_for(layout, SCHEDULE_SDD if mode == "sdd" else SCHEDULE_GROUP_WALK)
+    sched = schedule_for(layout, SCHEDULE_SDD) if mode == "sdd" else _group_walk_schedule(layout)
     with torch.cuda.device(a.device):
         stream = _k.current_stream()
         ws, ws_bytes = sched.workspace(_k.MODES[mode], batches, size_m, size_n, stream)

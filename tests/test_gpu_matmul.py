@@ -66,15 +66,15 @@ def test_split_groups_reuse_their_workspace(mode, ta, tb, dtype):
     library leaves zeroed: repeated calls, three 64-wide strips, several batches."""
     import sparse
     from sparse import _ops
-    old = _ops.SCHEDULE_GROUP_WALK
+    old = _ops.SCHEDULE_GROUP_WALK, _ops.SCHEDULE_GROUP_WALK_LONG
     try:
         for sched in ((2, 2), (4, 8), (3, 1)):
-            _ops.SCHEDULE_GROUP_WALK = sched
+            _ops.SCHEDULE_GROUP_WALK = _ops.SCHEDULE_GROUP_WALK_LONG = sched
             for name in ("long_row_5x40", "long_col_70x3"):
                 errs = [_run(mode, ZOO[name], 160, ta, tb, dtype, batch=(3,), seed=s) for s in range(3)]
                 assert max(errs) <= tol_of(dtype), (sched, name, errs)
     finally:
-        _ops.SCHEDULE_GROUP_WALK = old
+        _ops.SCHEDULE_GROUP_WALK, _ops.SCHEDULE_GROUP_WALK_LONG = old
 
 
 def test_split_result_is_deterministic():
