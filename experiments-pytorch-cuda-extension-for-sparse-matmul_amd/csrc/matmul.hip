@@ -4,11 +4,16 @@
 // unfinished fp16 twin sparse/native/sparse_hmm_gpu.cu:26-317.  Nothing of
 // their structure is kept: every nonzero 32x32 block is one MFMA tile owned by
 // ONE wavefront (v_mfma_f32_32x32x16_f16, fp32 accumulate; v_mfma_f32_32x32x2_f32
-// for fp32), operands whose contraction index is contiguous in memory go
-// straight from global memory into MFMA registers with 16-byte loads, operands
-// whose contraction index is the slow one pass through a wave-private LDS tile
-// and come back transposed with ds_read_b64_tr_b16.  No workgroup barrier sits
-// in any inner loop.
+// for fp32).  fp16 tiles are fetched with fully coalesced requests (lane l takes
+// 16-byte pieces l and l + 64 of a 2 KB tile, whatever its orientation), parked
+// in a wave-private, XOR-swizzled LDS tile and read back in MFMA layout:
+// ds_read_b128 when the contraction index is contiguous in the tile,
+// ds_read_b64_tr_b16 (hardware transpose) when it is the slow index.  MFMA-layout
+// loads straight from global memory (lane = row, 16 bytes at row stride) were
+// measured at a third of the coalesced rate and are only used by the fp32
+// kernels.  Data touched once (sparse blocks, results) moves with non-temporal
+// loads and stores; dense tiles, which are re-read out of L2, do not.  No
+// workgroup barrier sits in any inner loop.
 //
 // Work distribution: a schedule (see bsa.h) hands every wavefront a chunk of
 // consecutive table pairs of one group.  SDD: the chunk's blocks share the

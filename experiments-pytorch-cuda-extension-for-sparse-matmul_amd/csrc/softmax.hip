@@ -61,6 +61,15 @@ template <> struct Chunk<half_t> {
         hi = fmaxf((float)mx[0], (float)mx[1]);
         lo = fminf((float)mn[0], (float)mn[1]);
     }
+    // every element times f
+    static __device__ __forceinline__ uint4 scaled(const uint4 &r, float f)
+    {
+        float v[8];
+        unpack(r, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] *= f;
+        return pack(v);
+    }
     // element i := `fill` where col0 + i > limit
     static __device__ __forceinline__ void mask_right_of(uint4 &r, int col0, int limit, float fill)
     {
@@ -91,6 +100,14 @@ template <> struct Chunk<float> {
         unpack(r, v);
         hi = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
         lo = fminf(fminf(v[0], v[1]), fminf(v[2], v[3]));
+    }
+    static __device__ __forceinline__ uint4 scaled(const uint4 &r, float f)
+    {
+        float v[4];
+        unpack(r, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] *= f;
+        return pack(v);
     }
     static __device__ __forceinline__ void mask_right_of(uint4 &r, int col0, int limit, float fill)
     {
@@ -177,9 +194,9 @@ __device__ __forceinline__ float chunk_exp(const uint4 &raw, float scale2, float
     return sum;
 }
 
-// Hides a register from common-subexpression elimination: the second pass over a register-resident
-// slice must RE-derive the scaled scores from the packed data, not keep every unpacked float of the
-// first pass alive (that is 2-4x the registers of the slice itself).
+// Pins a value to its four packed registers: without it the compiler forwards the unpacked floats
+// of one pass over a register-resident slice to the next pass and keeps all of them alive (2-4x the
+// registers of the slice itself).
 __device__ __forceinline__ void launder(uint4 &r)
 {
     asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
@@ -189,11 +206,134 @@ __device__ __forceinline__ float finite_or_zero(float m) { return m == -__builti
 
 // ---------------------------------------------------------------------------
 // Row-sliced walk: a block row of at most CBS blocks goes whole to two wavefronts,
-// each owning 16 of the 32 element rows.  The wave issues every load of its slice
-// at once (one 16-byte request per lane and block for fp16), keeps the slice in
-// registers, and needs neither LDS nor a barrier: a row lives in LPR neighbouring
-// lanes.  NS = 16-byte chunks per lane and block of a slice.
+// each owning 16 of the 32 element rows, which it cuts into SUBS sub-slices of
+// R = 16 / SUBS element rows.  A sub-slice of one block is R * LPR lanes wide, so one
+// load instruction covers BPI = 64 / (R * LPR) consecutive blocks of the row.  The
+// wave issues every load of its slice at once, sub-slice by sub-slice, and then
+// finishes the sub-slices one after the other: while it computes and stores
+// sub-slice t the data of sub-slice t + 1 is still arriving, so loads, math and
+// stores overlap although all waves of the launch run in lockstep.  No LDS
+// storage and no barrier: a row lives in LPR neighbouring lanes of BPI lane groups.
+// The code is specialised on the number of load instructions per sub-slice, which
+// keeps every load unconditional (the wait counts the compiler derives are exact).
 // ---------------------------------------------------------------------------
+#ifndef BSA_SM_SUBS
+#define BSA_SM_SUBS 2
+#endif
+constexpr int SM_SUBS = BSA_SM_SUBS;
+
+template <int MASK>
+__device__ __forceinline__ float lane_xor(float x)
+{
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((lane_id() ^ MASK) << 2, __float_as_int(x)));
+}
+
+// all-reduce over the lanes that hold one element row of a sub-slice
+template <int LPR, int BPI, typename Op>
+__device__ __forceinline__ float slice_allreduce(float x, Op op)
+{
+    x = row_allreduce<LPR>(x, op);
+    if (BPI >= 2) x = op(x, lane_xor<32>(x));
+    if (BPI >= 4) x = op(x, lane_xor<16>(x));
+    return x;
+}
+
+template <typename T, int SUBS>
+struct SliceMap {
+    typedef Chunk<T> C;
+    static constexpr int R = BS / SCHED_ROW_SLICES / SUBS;   // element rows of a sub-slice
+    static constexpr int LPB = R * C::LPR;                    // lanes on one block's part of a sub-slice
+    static constexpr int BPI = WAVE / LPB;                    // blocks per load instruction
+    static constexpr int SUB_STRIDE = R * BS;                 // elements between sub-slices inside a block
+    static_assert(LPB <= WAVE && BPI <= 4, "sub-slice geometry");
+    int seg, row0, col0, lane_off;
+    __device__ __forceinline__ SliceMap(int slice)
+    {
+        const int l = lane_id();
+        seg = l / LPB;
+        row0 = (BS / SCHED_ROW_SLICES) * slice + (l % LPB) / C::LPR;      // + R * t
+        col0 = C::EPC * (l % C::LPR);
+        lane_off = (BS2 / SCHED_ROW_SLICES) * slice + (l % LPB) * C::EPC;  // + SUB_STRIDE * t, inside a block
+    }
+};
+
+template <typename T, int SUBS, int NI>
+__device__ __forceinline__ void softmax_fwd_sliced_body(const T *__restrict__ xb, T *__restrict__ yb,
+                                                        const DescWindow &win, const SchedEntry &e,
+                                                        float scale2, int causal)
+{
+    typedef Chunk<T> C;
+    typedef SliceMap<T, SUBS> Map;
+    constexpr int EPC = C::EPC, LPR = C::LPR, BPI = Map::BPI;
+    const Map map(e.part());
+    const int n = e.end - e.begin;
+    const float NEG_INF = -__builtin_inff();
+
+    // The table is row-major and idx is the row-major ordinal of a block, so pair p of the table
+    // IS block p of the operand and the blocks of a row lie one after the other in memory: the
+    // loads need nothing from the table (only the causal mask reads the block columns, which
+    // arrive while the data is in flight).  Lane's block of load instruction i is i * BPI + seg;
+    // lanes past the end of the row (last instruction only) load the last block instead, are
+    // masked out of the reductions and do not store.
+    const size_t row_off = (size_t)e.begin * BS2;
+    const T *xrow = xb + row_off;
+    T *yrow = yb + row_off;
+    const unsigned off = (unsigned)(map.seg * BS2 + map.lane_off);                        // + (i * BPI) * BS2 + t * SUB_STRIDE
+    const unsigned off_last = (unsigned)(min((NI - 1) * BPI + map.seg, n - 1) * BS2 + map.lane_off);
+    auto chunk_off = [&](int t, int i) {
+        return (i == NI - 1 ? off_last : off + (unsigned)(i * BPI * BS2)) + (unsigned)(t * Map::SUB_STRIDE);
+    };
+    uint4 raw[SUBS][NI];
+#pragma unroll
+    for (int t = 0; t < SUBS; ++t) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+            raw[t][i] = SM_ABLATE(16) ? make_uint4(off, i, t, map.col0) : ldg16_stream(xrow + chunk_off(t, i));
+        __builtin_amdgcn_sched_barrier(0);   // sub-slice t is requested in full before t + 1: it is needed first
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int t = 0; t < SUBS; ++t) {
+        const int row = map.row0 + t * Map::R;
+        float m = NEG_INF, s = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool tail = i == NI - 1 && n < NI * BPI;
+            const int last_col = win.get(e.begin + min(i * BPI + BPI - 1, n - 1)).col();
+            if (tail || (causal && last_col >= e.group)) {     // wave-uniform
+                const int j = i * BPI + map.seg;
+                const int pos = BPI == 1 ? win.get(e.begin + min(j, n - 1)).pos
+                                         : __builtin_amdgcn_ds_bpermute(min(j, n - 1) << 2, win.pos);
+                const int bcol = pos & 0xFFFF;
+                int limit = BS;                                 // last visible column inside the block
+                if (causal && bcol >= e.group) limit = bcol > e.group ? -1 : row;
+                if (j >= n) limit = -1;
+                const float fill = scale2 < 0.f ? __builtin_inff() : NEG_INF;   // -inf once scaled
+                C::mask_right_of(raw[t][i], map.col0, limit, fill);
+            }
+            m = fmaxf(m, chunk_scaled_max<T>(raw[t][i], scale2));
+        }
+        m = finite_or_zero(slice_allreduce<LPR, BPI>(m, MaxOp()));
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            float v[EPC];
+            s += chunk_exp<T>(raw[t][i], scale2, m, v);
+            raw[t][i] = C::pack(v);
+            launder(raw[t][i]);                  // park the exponentials PACKED: the compiler would keep 8 floats
+            __builtin_amdgcn_sched_barrier(0);   // one chunk at a time: unpacking them all at once spills
+        }
+        s = slice_allreduce<LPR, BPI>(s, AddOp());
+        s = s > 0.f ? 1.f / s : 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool mine = i < NI - 1 || i * BPI + map.seg < n;
+            if (mine && !SM_ABLATE(8)) stg16_stream(yrow + chunk_off(t, i), C::scaled(raw[t][i], s));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
 template <typename T, int CBS>
 __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *__restrict__ yb,
                                                    const BlockDesc *__restrict__ blocks, const SchedEntry &e,
@@ -202,82 +342,33 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
     typedef Chunk<T> C;
     constexpr int NS = C::NQ / SCHED_ROW_SLICES, EPC = C::EPC, LPR = C::LPR;
     constexpr int ROWS_PER_Q = WAVE / LPR;
+    constexpr int BPI = SliceMap<T, SM_SUBS>::BPI, NI_MAX = (CBS + BPI - 1) / BPI;
+    static_assert(NI_MAX <= 12, "add cases to the switch below");
     const int l = lane_id();
     const int n = e.end - e.begin;
-    const int row_base = (BS / SCHED_ROW_SLICES) * e.part() + l / LPR;   // + q * ROWS_PER_Q
-    const int col0 = EPC * (l % LPR);
-    const int slice_off = (BS2 / SCHED_ROW_SLICES) * e.part() + l * EPC;  // + q * 64 * EPC, inside a block
-    const float NEG_INF = -__builtin_inff();
-
-    float m[NS], s[NS];
-#pragma unroll
-    for (int q = 0; q < NS; ++q) { m[q] = NEG_INF; s[q] = 0.f; }
     DescWindow win;
     win.fetch(blocks, e.begin, e.end);
 
     if (n <= CBS) {
-        // block indices and columns are re-read from the window (v_readlane) in every pass:
-        // keeping 2 x CBS scalars alive would spill
-        uint4 raw[CBS][NS];
-#pragma unroll
-        for (int j = 0; j < CBS; ++j) {
-            if (j < n) {
-                const BlockDesc d = win.get(e.begin + j);
-#pragma unroll
-                for (int q = 0; q < NS; ++q)
-                    raw[j][q] = SM_ABLATE(16) ? make_uint4(d.idx, j, q, l)
-                                              : ldg16_stream(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC);
-            }
+#define BSA_SM_CASE(K) \
+    case K: if constexpr (K <= NI_MAX) softmax_fwd_sliced_body<T, SM_SUBS, K>(xb, yb, win, e, scale2, causal); break;
+        switch ((n + BPI - 1) / BPI) {
+            BSA_SM_CASE(1) BSA_SM_CASE(2) BSA_SM_CASE(3) BSA_SM_CASE(4) BSA_SM_CASE(5) BSA_SM_CASE(6)
+            BSA_SM_CASE(7) BSA_SM_CASE(8) BSA_SM_CASE(9) BSA_SM_CASE(10) BSA_SM_CASE(11) BSA_SM_CASE(12)
+            default: break;    // an empty row: nothing to write
         }
-#pragma unroll
-        for (int j = 0; j < CBS; ++j) {
-            if (j < n) {
-                const int bcol = win.get(e.begin + j).col();
-#pragma unroll
-                for (int q = 0; q < NS; ++q) {
-                    if (causal) mask_chunk<T>(raw[j][q], row_base + q * ROWS_PER_Q, col0, bcol, e.group, scale2);
-                    m[q] = fmaxf(m[q], chunk_scaled_max<T>(raw[j][q], scale2));
-                }
-            }
-        }
-#pragma unroll
-        for (int q = 0; q < NS; ++q) m[q] = finite_or_zero(row_allreduce<LPR>(m[q], MaxOp()));
-#pragma unroll
-        for (int j = 0; j < CBS; ++j) {
-            if (j < n) {
-#pragma unroll
-                for (int q = 0; q < NS; ++q) {
-                    float v[EPC];
-                    s[q] += chunk_exp<T>(raw[j][q], scale2, m[q], v);
-                    raw[j][q] = C::pack(v);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);   // one block at a time: unpacking them all at once spills
-        }
-#pragma unroll
-        for (int q = 0; q < NS; ++q) {
-            s[q] = row_allreduce<LPR>(s[q], AddOp());
-            s[q] = s[q] > 0.f ? 1.f / s[q] : 0.f;
-        }
-#pragma unroll
-        for (int j = 0; j < CBS; ++j) {
-            if (j < n) {
-#pragma unroll
-                for (int q = 0; q < NS; ++q) {
-                    float v[EPC];
-                    C::unpack(raw[j][q], v);
-#pragma unroll
-                    for (int i = 0; i < EPC; ++i) v[i] *= s[q];
-                    if (!SM_ABLATE(8) || v[0] == 1234.5f)
-                        stg16_stream(yb + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
+#undef BSA_SM_CASE
         return;
     }
 
     // longer than the register capacity (a schedule built with another slice_max): two passes
+    const int row_base = (BS / SCHED_ROW_SLICES) * e.part() + l / LPR;   // + q * ROWS_PER_Q
+    const int col0 = EPC * (l % LPR);
+    const int slice_off = (BS2 / SCHED_ROW_SLICES) * e.part() + l * EPC;  // + q * 64 * EPC, inside a block
+    const float NEG_INF = -__builtin_inff();
+    float m[NS], s[NS];
+#pragma unroll
+    for (int q = 0; q < NS; ++q) { m[q] = NEG_INF; s[q] = 0.f; }
     for (int p = e.begin; p < e.end; ++p) {
         if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
         const BlockDesc d = win.get(p);
@@ -324,7 +415,7 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
 // forward
 // ---------------------------------------------------------------------------
 template <typename T, int CB, int CBS>
-__global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
+__global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_eu(4))) void softmax_fwd_kernel(
     const T *__restrict__ x, T *__restrict__ y, const BlockDesc *__restrict__ blocks,
     const SchedEntry *__restrict__ sched, int n_swg, int batches, int nnz,
     float scale2 /* scale * log2(e) */, int causal)
@@ -504,6 +595,62 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_fwd_kernel(
 // ---------------------------------------------------------------------------
 // backward: dx = scale * (dy - sum_row(dy * y)) * y
 // ---------------------------------------------------------------------------
+// Row-sliced backward: the same sub-slice pipeline as the forward walk, over two inputs.
+template <typename T, int SUBS, int NI>
+__device__ __forceinline__ void softmax_bwd_sliced_body(const T *__restrict__ y, const T *__restrict__ dy,
+                                                        T *__restrict__ dx, const SchedEntry &e, float scale)
+{
+    typedef Chunk<T> C;
+    typedef SliceMap<T, SUBS> Map;
+    constexpr int EPC = C::EPC, LPR = C::LPR, BPI = Map::BPI;
+    const Map map(e.part());
+    const int n = e.end - e.begin;
+    const size_t row_off = (size_t)e.begin * BS2;     // pair p of the row-major table is block p of the operand
+    const unsigned off = (unsigned)(map.seg * BS2 + map.lane_off);
+    const unsigned off_last = (unsigned)(min((NI - 1) * BPI + map.seg, n - 1) * BS2 + map.lane_off);
+    auto chunk_off = [&](int t, int i) {
+        return (i == NI - 1 ? off_last : off + (unsigned)(i * BPI * BS2)) + (unsigned)(t * Map::SUB_STRIDE);
+    };
+    const bool mine_last = (NI - 1) * BPI + map.seg < n;   // lanes past the row's end load its last block again
+
+    uint4 ry[SUBS][NI], rd[SUBS][NI];
+#pragma unroll
+    for (int t = 0; t < SUBS; ++t) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            ry[t][i] = ldg16_stream(y + row_off + chunk_off(t, i));
+            rd[t][i] = ldg16_stream(dy + row_off + chunk_off(t, i));
+        }
+        __builtin_amdgcn_sched_barrier(0);   // sub-slice t is requested in full before t + 1: it is needed first
+    }
+#pragma unroll
+    for (int t = 0; t < SUBS; ++t) {
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            float a[EPC], b[EPC], part = 0.f;
+            C::unpack(ry[t][i], a);
+            C::unpack(rd[t][i], b);
+#pragma unroll
+            for (int k = 0; k < EPC; ++k) part += a[k] * b[k];
+            dot += (i < NI - 1 || mine_last) ? part : 0.f;
+        }
+        dot = slice_allreduce<LPR, BPI>(dot, AddOp());
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            float a[EPC], b[EPC];
+            launder(ry[t][i]);                // unpack again: the floats of the first pass are not kept
+            launder(rd[t][i]);
+            C::unpack(ry[t][i], a);
+            C::unpack(rd[t][i], b);
+#pragma unroll
+            for (int k = 0; k < EPC; ++k) a[k] = scale * (b[k] - dot) * a[k];
+            if (i < NI - 1 || mine_last) stg16_stream(dx + row_off + chunk_off(t, i), C::pack(a));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
 template <typename T, int CBS>
 __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, const T *__restrict__ dy,
                                                    T *__restrict__ dx, const BlockDesc *__restrict__ blocks,
@@ -511,8 +658,22 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
 {
     typedef Chunk<T> C;
     constexpr int NS = C::NQ / SCHED_ROW_SLICES, EPC = C::EPC, LPR = C::LPR;
+    constexpr int BPI = SliceMap<T, SM_SUBS>::BPI, NI_MAX = (CBS + BPI - 1) / BPI;
+    static_assert(NI_MAX <= 6, "add cases to the switch below");
     const int l = lane_id();
     const int n = e.end - e.begin;
+    if (n <= CBS) {
+#define BSA_SM_CASE(K) \
+    case K: if constexpr (K <= NI_MAX) softmax_bwd_sliced_body<T, SM_SUBS, K>(y, dy, dx, e, scale); break;
+        switch ((n + BPI - 1) / BPI) {
+            BSA_SM_CASE(1) BSA_SM_CASE(2) BSA_SM_CASE(3) BSA_SM_CASE(4) BSA_SM_CASE(5) BSA_SM_CASE(6)
+            default: break;    // an empty row: nothing to write
+        }
+#undef BSA_SM_CASE
+        return;
+    }
+
+    // longer than the register capacity (a schedule built with another slice_max): two passes
     const int slice_off = (BS2 / SCHED_ROW_SLICES) * e.part() + l * EPC;
     float dot[NS];
 #pragma unroll
@@ -535,36 +696,6 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
 #pragma unroll
         for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
     };
-
-    if (n <= CBS) {
-        uint4 ry[CBS][NS], rd[CBS][NS];
-#pragma unroll
-        for (int j = 0; j < CBS; ++j) {
-            if (j < n) {
-                const size_t o = (size_t)win.get(e.begin + j).idx * BS2 + slice_off;
-#pragma unroll
-                for (int q = 0; q < NS; ++q) {
-                    ry[j][q] = ldg16_stream(y + o + q * WAVE * EPC);
-                    rd[j][q] = ldg16_stream(dy + o + q * WAVE * EPC);
-                }
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < CBS; ++j)
-            if (j < n)
-#pragma unroll
-                for (int q = 0; q < NS; ++q) accumulate(ry[j][q], rd[j][q], q);
-#pragma unroll
-        for (int q = 0; q < NS; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
-#pragma unroll
-        for (int j = 0; j < CBS; ++j)
-            if (j < n)
-#pragma unroll
-                for (int q = 0; q < NS; ++q)
-                    stg16_stream(dx + (size_t)win.get(e.begin + j).idx * BS2 + slice_off + q * WAVE * EPC,
-                          finish(ry[j][q], rd[j][q], q));
-        return;
-    }
     for (int p = e.begin; p < e.end; ++p) {
         if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
         const size_t o = (size_t)win.get(p).idx * BS2 + slice_off;
@@ -583,7 +714,7 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
 }
 
 template <typename T, int CB, int CBS>
-__global__ __launch_bounds__(64 * SM_MAX_WAVES) void softmax_bwd_kernel(
+__global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_eu(4))) void softmax_bwd_kernel(
     const T *__restrict__ y, const T *__restrict__ dy, T *__restrict__ dx,
     const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
     int n_swg, int batches, int nnz, float scale)

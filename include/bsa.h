@@ -89,7 +89,8 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
  * With `slice_max` >= 0 (softmax only) a group of at most slice_max pairs is not
  * chunked at all: it goes whole to two wavefronts, each taking 16 of its 32
  * element rows (team word: waves = 1, part = slice, parts = 2), and these
- * wavefronts fill workgroups of their own at the front of the schedule.  Pass
+ * wavefronts fill workgroups of their own at the front of the schedule (slice_max
+ * <= 64).  Pass
  * -1 for the matmul schedules.
  * No counterpart in the reference, whose grids are (nnz, B) and
  * (B, M/32, N/32) (sparse/native/sparse_smm_gpu.cu:278-279).
