@@ -80,14 +80,17 @@ int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves)
     // waves: sum over parts of (len / cap + 1) <= nnz / cap + parts, parts <= nnz / (cap * waves) + groups;
     // first-fit padding wastes less than the waves it pads for
     int64_t slots = 2 * (2 * ((int64_t)nnz / cap) + groups + 1) + 2 * waves;
+    slots += 2 * (int64_t)groups;   // row-sliced groups take up to 4 slots each
     return slots + groups;   // one record per group in front
 }
 
 int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves, int allow_split, int slice_max,
-                       int32_t *sched, int64_t capacity, int32_t *counts_out, void *stream)
+                       int slices, int32_t *sched, int64_t capacity, int32_t *counts_out, void *stream)
 {
     if (slice_max < -1 || slice_max > 64)
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: slice_max %d outside [-1, 64]", slice_max);
+    if (slice_max >= 0 && slices != 2 && slices != 4)
+        return fail(BSA_ERR_INVALID, "bsa_schedule_build: slices must be 2 or 4, got %d", slices);
     if (!offsets || !sched || !counts_out) return fail(BSA_ERR_INVALID, "bsa_schedule_build: null pointer argument");
     if (groups < 1 || groups > 65535) return fail(BSA_ERR_INVALID, "bsa_schedule_build: %d groups outside [1, 65535]", groups);
     if (cap < 1) return fail(BSA_ERR_INVALID, "bsa_schedule_build: cap %d < 1", cap);
@@ -96,7 +99,7 @@ int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves, i
     if (capacity < 2 * ((int64_t)groups + 1) + waves + groups || capacity > (1LL << 28))
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: capacity %lld too small for %d groups (use bsa_schedule_capacity)",
                     (long long)capacity, groups);
-    return check_launch(bsa::launch_schedule_build(offsets, groups, cap, waves, allow_split != 0, slice_max, sched, capacity,
+    return check_launch(bsa::launch_schedule_build(offsets, groups, cap, waves, allow_split != 0, slice_max, slices, sched, capacity,
                                                    counts_out, (hipStream_t)stream),
                         "bsa_schedule_build");
 }

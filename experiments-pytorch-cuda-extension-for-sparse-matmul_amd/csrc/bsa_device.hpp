@@ -46,7 +46,6 @@ struct SchedEntry {
 };
 
 constexpr int SCHED_MAX_PARTS = 4095;
-constexpr int SCHED_ROW_SLICES = 2;   // a row-sliced group goes to 2 waves of 16 element rows each
 __host__ __device__ __forceinline__ int sched_team_word(int first_wave, int team_waves, int part, int parts)
 {
     return first_wave | (team_waves << 4) | (part << 8) | (int)((unsigned)parts << 20);

@@ -94,16 +94,16 @@ __global__ __launch_bounds__(LB_THREADS) void layout_build_kernel(
 struct GroupPlan {
     int parts;      // workgroup-sized pieces the group is cut into (or row slices, see below)
     int len;
-    bool sliced;    // the whole group goes to SCHED_ROW_SLICES waves, each taking some of its 32 element rows
+    bool sliced;    // the whole group goes to `slices` waves, each taking 32 / slices of its element rows
 };
 
-__device__ __forceinline__ GroupPlan plan_group(int len, int cap, int waves, int allow_split, int slice_max)
+__device__ __forceinline__ GroupPlan plan_group(int len, int cap, int waves, int allow_split, int slice_max, int slices)
 {
     GroupPlan p;
     p.len = len;
     p.sliced = len <= slice_max;
     if (p.sliced) {
-        p.parts = SCHED_ROW_SLICES;
+        p.parts = slices;
         return p;
     }
     const int span = cap * waves;                       // pairs one workgroup takes at the target chunk size
@@ -124,7 +124,7 @@ __device__ __forceinline__ int waves_of_part(int part_len, int cap, int waves)
 }
 
 __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
-    const int *__restrict__ offsets, int groups, int cap, int waves, int allow_split, int slice_max,
+    const int *__restrict__ offsets, int groups, int cap, int waves, int allow_split, int slice_max, int slices,
     int4 *__restrict__ sched, int slot_capacity, int *__restrict__ counts_out)
 {
     __shared__ int total_slots;
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
         int pos = 0, tile_slots = 0, split_groups = 0;
         for (int pass = 0; pass < 2; ++pass) {
             for (int g = 0; g < groups; ++g) {
-                const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split, slice_max);
+                const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split, slice_max, slices);
                 if (gp.sliced != (pass == 0)) continue;
                 if (gp.sliced) {
                     meta[g] = make_int4(pos, -1, -1, gp.parts);
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
         }
         int n_wgs = (pos + waves - 1) / waves;
         total_slots = n_wgs * waves;
-        counts_out[0] = n_wgs;
+        counts_out[0] = total_slots <= slot_capacity ? n_wgs : -1;   // -1: the table is too small, nothing usable
         counts_out[1] = tile_slots;
         counts_out[2] = split_groups;
         counts_out[3] = pos;
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
     __syncthreads();
     for (int g = tid; g < groups; g += LB_THREADS) {
         const int lo = offsets[g];
-        const GroupPlan gp = plan_group(offsets[g + 1] - lo, cap, waves, allow_split, slice_max);
+        const GroupPlan gp = plan_group(offsets[g + 1] - lo, cap, waves, allow_split, slice_max, slices);
         int pos = meta[g].x;
         if (gp.sliced) {
             for (int t = 0; t < gp.parts; ++t)
@@ -210,10 +210,10 @@ hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_b
 }
 
 hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                                 int allow_split, int slice_max, int32_t *sched, int64_t capacity,
+                                 int allow_split, int slice_max, int slices, int32_t *sched, int64_t capacity,
                                  int32_t *counts_out, hipStream_t stream)
 {
-    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, allow_split, slice_max,
+    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, allow_split, slice_max, slices,
                                                        (int4 *)sched, (int)(capacity - groups),
                                                        counts_out);
     return hipGetLastError();

@@ -205,9 +205,9 @@ __device__ __forceinline__ void launder(uint4 &r)
 __device__ __forceinline__ float finite_or_zero(float m) { return m == -__builtin_inff() ? 0.f : m; }
 
 // ---------------------------------------------------------------------------
-// Row-sliced walk: a block row of at most CBS blocks goes whole to two wavefronts,
-// each owning 16 of the 32 element rows, which it cuts into SUBS sub-slices of
-// R = 16 / SUBS element rows.  A sub-slice of one block is R * LPR lanes wide, so one
+// Row-sliced walk: a block row of at most CBS blocks goes whole to SLICES wavefronts,
+// each owning 32 / SLICES of the 32 element rows, which it cuts into SUBS sub-slices of
+// R = 32 / SLICES / SUBS element rows.  A sub-slice of one block is R * LPR lanes wide, so one
 // load instruction covers BPI = 64 / (R * LPR) consecutive blocks of the row.  The
 // wave issues every load of its slice at once, sub-slice by sub-slice, and then
 // finishes the sub-slices one after the other: while it computes and stores
@@ -221,6 +221,11 @@ __device__ __forceinline__ float finite_or_zero(float m) { return m == -__builti
 #define BSA_SM_SUBS 2
 #endif
 constexpr int SM_SUBS = BSA_SM_SUBS;
+#ifndef BSA_SM_FWD_SLICES
+#define BSA_SM_FWD_SLICES 4
+#endif
+constexpr int SM_FWD_SLICES = BSA_SM_FWD_SLICES;   // slices the register-resident walks are compiled for
+constexpr int SM_BWD_SLICES = 4;
 
 template <int MASK>
 __device__ __forceinline__ float lane_xor(float x)
@@ -238,10 +243,10 @@ __device__ __forceinline__ float slice_allreduce(float x, Op op)
     return x;
 }
 
-template <typename T, int SUBS>
+template <typename T, int SLICES, int SUBS>
 struct SliceMap {
     typedef Chunk<T> C;
-    static constexpr int R = BS / SCHED_ROW_SLICES / SUBS;   // element rows of a sub-slice
+    static constexpr int R = BS / SLICES / SUBS;              // element rows of a sub-slice
     static constexpr int LPB = R * C::LPR;                    // lanes on one block's part of a sub-slice
     static constexpr int BPI = WAVE / LPB;                    // blocks per load instruction
     static constexpr int SUB_STRIDE = R * BS;                 // elements between sub-slices inside a block
@@ -251,19 +256,19 @@ struct SliceMap {
     {
         const int l = lane_id();
         seg = l / LPB;
-        row0 = (BS / SCHED_ROW_SLICES) * slice + (l % LPB) / C::LPR;      // + R * t
+        row0 = (BS / SLICES) * slice + (l % LPB) / C::LPR;      // + R * t
         col0 = C::EPC * (l % C::LPR);
-        lane_off = (BS2 / SCHED_ROW_SLICES) * slice + (l % LPB) * C::EPC;  // + SUB_STRIDE * t, inside a block
+        lane_off = (BS2 / SLICES) * slice + (l % LPB) * C::EPC;  // + SUB_STRIDE * t, inside a block
     }
 };
 
-template <typename T, int SUBS, int NI>
+template <typename T, int SLICES, int SUBS, int NI>
 __device__ __forceinline__ void softmax_fwd_sliced_body(const T *__restrict__ xb, T *__restrict__ yb,
                                                         const DescWindow &win, const SchedEntry &e,
                                                         float scale2, int causal)
 {
     typedef Chunk<T> C;
-    typedef SliceMap<T, SUBS> Map;
+    typedef SliceMap<T, SLICES, SUBS> Map;
     constexpr int EPC = C::EPC, LPR = C::LPR, BPI = Map::BPI;
     const Map map(e.part());
     const int n = e.end - e.begin;
@@ -334,24 +339,43 @@ __device__ __forceinline__ void softmax_fwd_sliced_body(const T *__restrict__ xb
     }
 }
 
-template <typename T, int CBS>
+// Lane map of whole blocks with a row filter, for sliced rows that the register-resident walk
+// does not take (longer than its capacity, or cut into another number of slices): chunk q of a
+// lane belongs to the wave when its element row lies in the wave's slice.
+template <typename T>
+struct SliceFilter {
+    typedef Chunk<T> C;
+    static constexpr int ROWS_PER_Q = WAVE / C::LPR;
+    int row0, col0, lo, hi;
+    __device__ __forceinline__ SliceFilter(const SchedEntry &e)
+    {
+        const int l = lane_id(), rows = BS / e.parts();
+        row0 = l / C::LPR;
+        col0 = C::EPC * (l % C::LPR);
+        lo = rows * e.part();
+        hi = lo + rows;
+    }
+    __device__ __forceinline__ int row(int q) const { return row0 + q * ROWS_PER_Q; }
+    __device__ __forceinline__ bool mine(int q) const { return row(q) >= lo && row(q) < hi; }
+};
+
+template <typename T, int CBS, int SLICES>
 __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *__restrict__ yb,
                                                    const BlockDesc *__restrict__ blocks, const SchedEntry &e,
                                                    float scale2, int causal)
 {
     typedef Chunk<T> C;
-    constexpr int NS = C::NQ / SCHED_ROW_SLICES, EPC = C::EPC, LPR = C::LPR;
-    constexpr int ROWS_PER_Q = WAVE / LPR;
-    constexpr int BPI = SliceMap<T, SM_SUBS>::BPI, NI_MAX = (CBS + BPI - 1) / BPI;
+    constexpr int NQ = C::NQ, EPC = C::EPC, LPR = C::LPR;
+    constexpr int BPI = SliceMap<T, SLICES, SM_SUBS>::BPI, NI_MAX = (CBS + BPI - 1) / BPI;
     static_assert(NI_MAX <= 12, "add cases to the switch below");
     const int l = lane_id();
     const int n = e.end - e.begin;
     DescWindow win;
     win.fetch(blocks, e.begin, e.end);
 
-    if (n <= CBS) {
+    if (e.parts() == SLICES && n <= CBS) {
 #define BSA_SM_CASE(K) \
-    case K: if constexpr (K <= NI_MAX) softmax_fwd_sliced_body<T, SM_SUBS, K>(xb, yb, win, e, scale2, causal); break;
+    case K: if constexpr (K <= NI_MAX) softmax_fwd_sliced_body<T, SLICES, SM_SUBS, K>(xb, yb, win, e, scale2, causal); break;
         switch ((n + BPI - 1) / BPI) {
             BSA_SM_CASE(1) BSA_SM_CASE(2) BSA_SM_CASE(3) BSA_SM_CASE(4) BSA_SM_CASE(5) BSA_SM_CASE(6)
             BSA_SM_CASE(7) BSA_SM_CASE(8) BSA_SM_CASE(9) BSA_SM_CASE(10) BSA_SM_CASE(11) BSA_SM_CASE(12)
@@ -361,22 +385,21 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
         return;
     }
 
-    // longer than the register capacity (a schedule built with another slice_max): two passes
-    const int row_base = (BS / SCHED_ROW_SLICES) * e.part() + l / LPR;   // + q * ROWS_PER_Q
-    const int col0 = EPC * (l % LPR);
-    const int slice_off = (BS2 / SCHED_ROW_SLICES) * e.part() + l * EPC;  // + q * 64 * EPC, inside a block
+    // two passes over global memory: online (max, sum), then normalise
+    const SliceFilter<T> f(e);
     const float NEG_INF = -__builtin_inff();
-    float m[NS], s[NS];
+    float m[NQ], s[NQ];
 #pragma unroll
-    for (int q = 0; q < NS; ++q) { m[q] = NEG_INF; s[q] = 0.f; }
+    for (int q = 0; q < NQ; ++q) { m[q] = NEG_INF; s[q] = 0.f; }
     for (int p = e.begin; p < e.end; ++p) {
         if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
         const BlockDesc d = win.get(p);
 #pragma unroll
-        for (int q = 0; q < NS; ++q) {
+        for (int q = 0; q < NQ; ++q) {
+            if (!f.mine(q)) continue;
             float v[EPC];
-            scaled_chunk<T>(ldg16_stream(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
-                            row_base + q * ROWS_PER_Q, col0, d.col(), e.group, scale2, causal, v);
+            scaled_chunk<T>(ldg16_stream(xb + (size_t)d.idx * BS2 + (l + WAVE * q) * EPC),
+                            f.row(q), f.col0, d.col(), e.group, scale2, causal, v);
             float bm = v[0];
 #pragma unroll
             for (int i = 1; i < EPC; ++i) bm = fmaxf(bm, v[i]);
@@ -390,7 +413,7 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
         }
     }
 #pragma unroll
-    for (int q = 0; q < NS; ++q) {
+    for (int q = 0; q < NQ; ++q) {      // all lanes take part in the exchange; rows of other slices carry (-inf, 0)
         const float rm = finite_or_zero(row_allreduce<LPR>(m[q], MaxOp()));
         s[q] = row_allreduce<LPR>(s[q] * exp2_fast(m[q] - rm), AddOp());
         s[q] = s[q] > 0.f ? 1.f / s[q] : 0.f;
@@ -400,13 +423,14 @@ __device__ __forceinline__ void softmax_fwd_sliced(const T *__restrict__ xb, T *
         if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
         const BlockDesc d = win.get(p);
 #pragma unroll
-        for (int q = 0; q < NS; ++q) {
+        for (int q = 0; q < NQ; ++q) {
+            if (!f.mine(q)) continue;
             float v[EPC];
-            scaled_chunk<T>(ldg16_stream(xb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC),
-                            row_base + q * ROWS_PER_Q, col0, d.col(), e.group, scale2, causal, v);
+            scaled_chunk<T>(ldg16_stream(xb + (size_t)d.idx * BS2 + (l + WAVE * q) * EPC),
+                            f.row(q), f.col0, d.col(), e.group, scale2, causal, v);
 #pragma unroll
             for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - m[q]) * s[q];
-            stg16_stream(yb + (size_t)d.idx * BS2 + slice_off + q * WAVE * EPC, C::pack(v));
+            stg16_stream(yb + (size_t)d.idx * BS2 + (l + WAVE * q) * EPC, C::pack(v));
         }
     }
 }
@@ -438,7 +462,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
     // Row-sliced waves fill workgroups of their own (the schedule builder sees to that), so this
     // branch is uniform over the workgroup and the barrier below is never left waiting.
     if (active && e.parts() > 1) {
-        softmax_fwd_sliced<T, CBS>(xb, yb, blocks, e, scale2, causal);
+        softmax_fwd_sliced<T, CBS, SM_FWD_SLICES>(xb, yb, blocks, e, scale2, causal);
         return;
     }
     if (sched[swg * W].parts() > 1) return;   // an unused slot behind the last row-sliced waves
@@ -596,12 +620,12 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
 // backward: dx = scale * (dy - sum_row(dy * y)) * y
 // ---------------------------------------------------------------------------
 // Row-sliced backward: the same sub-slice pipeline as the forward walk, over two inputs.
-template <typename T, int SUBS, int NI>
+template <typename T, int SLICES, int SUBS, int NI>
 __device__ __forceinline__ void softmax_bwd_sliced_body(const T *__restrict__ y, const T *__restrict__ dy,
                                                         T *__restrict__ dx, const SchedEntry &e, float scale)
 {
     typedef Chunk<T> C;
-    typedef SliceMap<T, SUBS> Map;
+    typedef SliceMap<T, SLICES, SUBS> Map;
     constexpr int EPC = C::EPC, LPR = C::LPR, BPI = Map::BPI;
     const Map map(e.part());
     const int n = e.end - e.begin;
@@ -651,20 +675,20 @@ __device__ __forceinline__ void softmax_bwd_sliced_body(const T *__restrict__ y,
     }
 }
 
-template <typename T, int CBS>
+template <typename T, int CBS, int SLICES>
 __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, const T *__restrict__ dy,
                                                    T *__restrict__ dx, const BlockDesc *__restrict__ blocks,
                                                    const SchedEntry &e, float scale)
 {
     typedef Chunk<T> C;
-    constexpr int NS = C::NQ / SCHED_ROW_SLICES, EPC = C::EPC, LPR = C::LPR;
-    constexpr int BPI = SliceMap<T, SM_SUBS>::BPI, NI_MAX = (CBS + BPI - 1) / BPI;
+    constexpr int NQ = C::NQ, EPC = C::EPC, LPR = C::LPR;
+    constexpr int BPI = SliceMap<T, SLICES, SM_SUBS>::BPI, NI_MAX = (CBS + BPI - 1) / BPI;
     static_assert(NI_MAX <= 6, "add cases to the switch below");
     const int l = lane_id();
     const int n = e.end - e.begin;
-    if (n <= CBS) {
+    if (e.parts() == SLICES && n <= CBS) {
 #define BSA_SM_CASE(K) \
-    case K: if constexpr (K <= NI_MAX) softmax_bwd_sliced_body<T, SM_SUBS, K>(y, dy, dx, e, scale); break;
+    case K: if constexpr (K <= NI_MAX) softmax_bwd_sliced_body<T, SLICES, SM_SUBS, K>(y, dy, dx, e, scale); break;
         switch ((n + BPI - 1) / BPI) {
             BSA_SM_CASE(1) BSA_SM_CASE(2) BSA_SM_CASE(3) BSA_SM_CASE(4) BSA_SM_CASE(5) BSA_SM_CASE(6)
             default: break;    // an empty row: nothing to write
@@ -673,43 +697,40 @@ __device__ __forceinline__ void softmax_bwd_sliced(const T *__restrict__ y, cons
         return;
     }
 
-    // longer than the register capacity (a schedule built with another slice_max): two passes
-    const int slice_off = (BS2 / SCHED_ROW_SLICES) * e.part() + l * EPC;
-    float dot[NS];
+    // two passes over global memory (see SliceFilter)
+    const SliceFilter<T> f(e);
+    float dot[NQ];
 #pragma unroll
-    for (int q = 0; q < NS; ++q) dot[q] = 0.f;
+    for (int q = 0; q < NQ; ++q) dot[q] = 0.f;
     DescWindow win;
-    win.fetch(blocks, e.begin, e.end);
-
-    auto finish = [&](const uint4 &uy, const uint4 &ud, int q) {
-        float a[EPC], b[EPC];
-        C::unpack(uy, a);
-        C::unpack(ud, b);
-#pragma unroll
-        for (int i = 0; i < EPC; ++i) a[i] = scale * (b[i] - dot[q]) * a[i];
-        return C::pack(a);
-    };
-    auto accumulate = [&](const uint4 &uy, const uint4 &ud, int q) {
-        float a[EPC], b[EPC];
-        C::unpack(uy, a);
-        C::unpack(ud, b);
-#pragma unroll
-        for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
-    };
-    for (int p = e.begin; p < e.end; ++p) {
-        if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
-        const size_t o = (size_t)win.get(p).idx * BS2 + slice_off;
-#pragma unroll
-        for (int q = 0; q < NS; ++q) accumulate(ldg16_stream(y + o + q * WAVE * EPC), ldg16_stream(dy + o + q * WAVE * EPC), q);
-    }
-#pragma unroll
-    for (int q = 0; q < NS; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
     for (int p = e.begin; p < e.end; ++p) {
         if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
-        const size_t o = (size_t)win.get(p).idx * BS2 + slice_off;
+        const size_t o = (size_t)win.get(p).idx * BS2;
 #pragma unroll
-        for (int q = 0; q < NS; ++q)
-            stg16_stream(dx + o + q * WAVE * EPC, finish(ldg16_stream(y + o + q * WAVE * EPC), ldg16_stream(dy + o + q * WAVE * EPC), q));
+        for (int q = 0; q < NQ; ++q) {
+            if (!f.mine(q)) continue;
+            float a[EPC], b[EPC];
+            C::unpack(ldg16_stream(y + o + (l + WAVE * q) * EPC), a);
+            C::unpack(ldg16_stream(dy + o + (l + WAVE * q) * EPC), b);
+#pragma unroll
+            for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) dot[q] = row_allreduce<LPR>(dot[q], AddOp());
+    for (int p = e.begin; p < e.end; ++p) {
+        if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
+        const size_t o = (size_t)win.get(p).idx * BS2;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            if (!f.mine(q)) continue;
+            float a[EPC], b[EPC];
+            C::unpack(ldg16_stream(y + o + (l + WAVE * q) * EPC), a);
+            C::unpack(ldg16_stream(dy + o + (l + WAVE * q) * EPC), b);
+#pragma unroll
+            for (int i = 0; i < EPC; ++i) a[i] = scale * (b[i] - dot[q]) * a[i];
+            stg16_stream(dx + o + (l + WAVE * q) * EPC, C::pack(a));
+        }
     }
 }
 
@@ -735,7 +756,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
     const int row0 = l / LPR;
 
     if (active && e.parts() > 1) {   // row-sliced waves sit in workgroups of their own
-        softmax_bwd_sliced<T, CBS>(y + boff, dy + boff, dx + boff, blocks, e, scale);
+        softmax_bwd_sliced<T, CBS, SM_BWD_SLICES>(y + boff, dy + boff, dx + boff, blocks, e, scale);
         return;
     }
     if (sched[swg * W].parts() > 1) return;
@@ -847,11 +868,11 @@ hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t s
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
     const float scale2 = p.scale * 1.4426950408889634f;
     if (dtype == BSA_F16)
-        softmax_fwd_kernel<half_t, 4, 24><<<grid, block, 0, st>>>(
+        softmax_fwd_kernel<half_t, 4, 48><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (half_t *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
     else
-        softmax_fwd_kernel<float, 2, 12><<<grid, block, 0, st>>>(
+        softmax_fwd_kernel<float, 2, 24><<<grid, block, 0, st>>>(
             (const float *)p.x, (float *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
     return hipGetLastError();
@@ -861,11 +882,11 @@ hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t 
 {
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
     if (dtype == BSA_F16)
-        softmax_bwd_kernel<half_t, 2, 12><<<grid, block, 0, st>>>(
+        softmax_bwd_kernel<half_t, 2, 24><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (const half_t *)p.dy, (half_t *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     else
-        softmax_bwd_kernel<float, 1, 6><<<grid, block, 0, st>>>(
+        softmax_bwd_kernel<float, 1, 12><<<grid, block, 0, st>>>(
             (const float *)p.x, (const float *)p.dy, (float *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     return hipGetLastError();

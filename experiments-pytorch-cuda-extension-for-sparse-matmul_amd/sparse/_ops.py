@@ -16,9 +16,11 @@ SCHEDULE_GROUP_WALK_LONG = (8, 4)    # tables with longer groups (columns of cau
 GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
-# block rows of at most this many blocks are handed whole to two wavefronts (16 element rows each),
-# which keep them in registers and need no exchange; per dtype: forward, backward
-SOFTMAX_SLICE_MAX = {torch.float16: (24, 12), torch.float32: (12, 6)}
+# block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
+# each), which keep them in registers and need no exchange; per dtype: forward, backward (the
+# backward walk keeps two inputs)
+SOFTMAX_SLICE_MAX = {torch.float16: (48, 24), torch.float32: (24, 12)}
+SOFTMAX_SLICES = (4, 4)              # forward, backward
 
 _DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
 
@@ -27,16 +29,18 @@ class Schedule:
     """Device-resident wavefront schedule of one offset table."""
 
     def __init__(self, offsets: torch.Tensor, nnz: int, cap: int, waves: int, allow_split: bool = True,
-                 slice_max: int = -1):
+                 slice_max: int = -1, slices: int = 2):
         groups = offsets.numel() - 1
         capacity = _k.lib.bsa_schedule_capacity(groups, nnz, cap, waves)
         self.table = torch.empty(4 * capacity, dtype=torch.int32, device=offsets.device)
         counts = torch.empty(4, dtype=torch.int32, device=offsets.device)
         with torch.cuda.device(offsets.device):
             _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves, int(allow_split), slice_max,
-                                               self.table.data_ptr(), capacity, counts.data_ptr(),
+                                               slices, self.table.data_ptr(), capacity, counts.data_ptr(),
                                                _k.current_stream()))
         self.workgroups, self.tile_slots, self.split_groups, self.slots = (int(v) for v in counts.tolist())
+        if self.workgroups < 0:
+            raise _k.BsaError("schedule table too small for this offset table")
         self.groups = groups
         self.waves = waves
         self.cap = cap
@@ -85,7 +89,8 @@ def _group_walk_schedule(layout):
 
 def _softmax_schedule(layout, dtype, backward):
     cap, waves = SCHEDULE_SOFTMAX
-    return schedule_for(layout, (cap, waves, False, SOFTMAX_SLICE_MAX[dtype][1 if backward else 0]))
+    which = 1 if backward else 0
+    return schedule_for(layout, (cap, waves, False, SOFTMAX_SLICE_MAX[dtype][which], SOFTMAX_SLICES[which]))
 
 
 def _check_layout(layout, name):

@@ -28,7 +28,7 @@ SIGNATURES = {
     "bsa_layout_workspace_bytes": (ctypes.c_size_t, [_i, _i]),
     "bsa_layout_build": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bsa_schedule_capacity": (_i64, [_i, _i, _i, _i]),
-    "bsa_schedule_build": (_i, [_vp, _i, _i, _i, _i, _i, _vp, _i64, _vp, _vp]),
+    "bsa_schedule_build": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _vp]),
     "bsa_matmul_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i, _i, _i, _i]),
     "bsa_matmul": (_i, [_i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp, ctypes.c_size_t,
                         _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),

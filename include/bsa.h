@@ -86,22 +86,25 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
  * most that many pairs when `allow_split` != 0 (matmul), and gets longer
  * chunks otherwise (softmax, whose rows cannot be split across workgroups).
  * Empty groups get one wavefront with an empty chunk (it writes the zeros).
- * With `slice_max` >= 0 (softmax only) a group of at most slice_max pairs is not
- * chunked at all: it goes whole to two wavefronts, each taking 16 of its 32
- * element rows (team word: waves = 1, part = slice, parts = 2), and these
- * wavefronts fill workgroups of their own at the front of the schedule (slice_max
- * <= 64).  Pass
- * -1 for the matmul schedules.
+ * With `slice_max` >= 0 (softmax only, at most 64) a group of at most slice_max
+ * pairs is not chunked at all: it goes whole to `slices` wavefronts (2 or 4),
+ * each taking 32 / slices of its 32 element rows (team word: waves = 1, part =
+ * slice, parts = slices), and these wavefronts fill workgroups of their own at
+ * the front of the schedule.  The softmax kernels keep such a slice in registers
+ * when slices is 4 and the group has at most 48 (fp16) / 24 (fp32) pairs in the
+ * forward and 24 / 12 pairs in the backward kernel; other sliced groups are
+ * still computed correctly, by a slower two-pass walk.  Pass slice_max = -1 for the matmul schedules.
  * No counterpart in the reference, whose grids are (nnz, B) and
  * (B, M/32, N/32) (sparse/native/sparse_smm_gpu.cu:278-279).
  *   sched        device int32[4 * bsa_schedule_capacity(...)]
- *   counts_out   device int32[4]: workgroups the schedule uses, partial-tile
+ *   counts_out   device int32[4]: workgroups the schedule uses (-1 if `capacity`
+ *                was too small: the table is then unusable), partial-tile
  *                slots, split groups, wavefront slots in use
  */
 int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves);
 int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                       int allow_split, int slice_max, int32_t *sched, int64_t capacity,
-                       int32_t *counts_out, void *stream);
+                       int allow_split, int slice_max, int slices, int32_t *sched,
+                       int64_t capacity, int32_t *counts_out, void *stream);
 
 /* ---- block-sparse matmul -----------------------------------------------
  * Replaces sparse_matmul's launch half: sparse_smm_32x32x32_kernel_wrapper and

@@ -83,9 +83,11 @@ def test_other_entry_points_validate(k):
     assert k.lib.bsa_layout_build(None, 4, 4, P, P, P, P, P, P, None) == -1
     assert k.lib.bsa_layout_build(P, 40000, 4, P, P, P, P, P, P, None) == -1
     assert "32767" in k.lib.bsa_last_error().decode()
-    assert k.lib.bsa_schedule_build(P, 4, 0, 4, 1, -1, P, 100, P, None) == -1
-    assert k.lib.bsa_schedule_build(P, 4, 4, 4, 1, -1, P, 3, P, None) == -1
+    assert k.lib.bsa_schedule_build(P, 4, 0, 4, 1, -1, 2, P, 100, P, None) == -1
+    assert k.lib.bsa_schedule_build(P, 4, 4, 4, 1, -1, 2, P, 3, P, None) == -1
     assert "capacity" in k.lib.bsa_last_error().decode()
+    assert k.lib.bsa_schedule_build(P, 4, 4, 4, 0, 8, 3, P, 100, P, None) == -1
+    assert "slices" in k.lib.bsa_last_error().decode()
     assert k.lib.bsa_softmax_forward(3, P, P, P, P, P, 1, 4, 4, 4, 5, 1, 1.0, 0, None) == -3
     assert k.lib.bsa_softmax_forward(1, P, None, P, P, P, 1, 4, 4, 4, 5, 1, 1.0, 0, None) == -1
     assert k.lib.bsa_softmax_backward(1, P, P, P, P, P, P, 1, 4, 4, 4, 5, 0, 1.0, None) == -1

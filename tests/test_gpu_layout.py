@@ -128,17 +128,17 @@ def test_schedule_covers_every_pair_once(name, mask, cap, waves, split):
 
 
 @pytest.mark.parametrize("name,mask", _more_masks())
-@pytest.mark.parametrize("cap,waves,slice_max", [(4, 4, 24), (4, 4, 3), (2, 2, 0), (4, 8, 64)])
-def test_row_sliced_schedule(name, mask, cap, waves, slice_max):
-    """Softmax schedules with slice_max: a short row goes whole to two wavefronts (slices 0 and 1 of
-    its element rows) that sit in one workgroup among other sliced rows at the front of the
-    schedule; every other row is chunked as without slicing and never split into parts."""
+@pytest.mark.parametrize("cap,waves,slice_max,slices", [(4, 4, 24, 2), (4, 4, 3, 4), (2, 2, 0, 2), (4, 8, 64, 4)])
+def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices):
+    """Softmax schedules with slice_max: a short row goes whole to `slices` wavefronts (one slice of
+    its element rows each) that sit among other sliced rows at the front of the schedule; every
+    other row is chunked as without slicing and never split into parts."""
     from sparse import _ops
     mask = np.asarray(mask)
     L = _layout(mask)
     offs = L.row_layout[1].cpu().numpy()
     groups = len(offs) - 1
-    s = _ops.Schedule(L.row_layout[1], L.num_blocks, cap, waves, False, slice_max)
+    s = _ops.Schedule(L.row_layout[1], L.num_blocks, cap, waves, False, slice_max, slices)
     raw = s.table.cpu().numpy().reshape(-1, 4)
     meta, tab = raw[:groups], raw[groups: groups + s.workgroups * waves]
     assert (s.tile_slots, s.split_groups) == (0, 0)
@@ -153,7 +153,7 @@ def test_row_sliced_schedule(name, mask, cap, waves, slice_max):
         first, nw, part, parts = team & 0xF, (team >> 4) & 0xF, (team >> 8) & 0xFFF, team >> 20
         wg, in_wg = divmod(slot, waves)
         if g in slices_seen:
-            assert (b, e) == (offs[g], offs[g + 1]) and nw == 1 and parts == 2 and first == in_wg
+            assert (b, e) == (offs[g], offs[g + 1]) and nw == 1 and parts == slices and first == in_wg
             slices_seen[g].append((wg, part))
             last_sliced_wg = max(last_sliced_wg, wg)
         else:
@@ -163,7 +163,7 @@ def test_row_sliced_schedule(name, mask, cap, waves, slice_max):
             assert meta[g][0] == groups * 0 + (wg * waves + first)
     for g in sliced:
         got = sorted(slices_seen[g])
-        assert [p for _, p in got] == [0, 1] and got[0][0] == got[1][0], (g, got)   # both slices, one workgroup
+        assert sorted(p for _, p in got) == list(range(slices)), (g, got)            # every slice once
         covered[offs[g]: offs[g + 1]] += 1
     assert np.all(covered[: int(offs[-1])] == 1)
     assert last_sliced_wg < first_other_wg                      # sliced rows fill workgroups of their own, first

@@ -115,3 +115,56 @@ def test_backward_long_rows():
     from sparse.kernel import sparse_ops
     dx = sparse_ops.sparse_softmax_backward(y.cuda(), dy.cuda(), L.row_layout[0], L.row_layout[1], 0.5)
     assert rel_err(to_np(dx), so.backward(to_np(y), to_np(dy), mask, 0.5)) <= 2e-3
+
+
+def _tri(n):
+    return np.tril(np.ones((n, n), dtype=np.int64))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_every_row_length_up_to_50(dtype, causal):
+    """Lower-triangular mask: row r has r + 1 blocks, so every specialisation of the register-resident
+    walk (1..48 blocks: lanes past the row's end in every position) and the first team rows are hit."""
+    y, ref = _fwd(_tri(50), dtype, 0.125, causal, batch=(2,), std=2.0, seed=5)
+    assert np.all(np.isfinite(y))
+    assert rel_err(y, ref) <= tol_of(dtype)
+    rows = y.reshape(2, -1, 32, 32).sum(axis=-1)            # per block: sum over its columns
+    offs = lo.create_layout(_tri(50))[1]
+    for r in range(50):
+        assert np.allclose(rows[:, offs[r]:offs[r + 1]].sum(axis=1), 1.0, atol=5e-3 if dtype == torch.float16 else 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_backward_every_row_length_up_to_26(dtype):
+    import sparse
+    from sparse.kernel import sparse_ops
+    mask = _tri(26)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    g = torch.Generator().manual_seed(3)
+    y = torch.rand(2, L.num_blocks, 32, 32, generator=g).to(dtype)
+    dy = torch.randn(2, L.num_blocks, 32, 32, generator=g).to(dtype)
+    dx = sparse_ops.sparse_softmax_backward(y.cuda(), dy.cuda(), L.row_layout[0], L.row_layout[1], 0.25)
+    assert rel_err(to_np(dx), so.backward(to_np(y), to_np(dy), mask, 0.25)) <= tol_of(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("slice_max,slices", [(64, 2), (64, 4), (5, 4), (5, 2), (-1, 2)])
+def test_schedules_the_resident_walk_does_not_take(monkeypatch, dtype, slice_max, slices):
+    """Sliced rows longer than the register capacity, or cut into another number of slices than the
+    kernel keeps in registers, go through the two-pass walk and give the same result."""
+    import sparse
+    from sparse import _ops
+    from sparse.kernel import sparse_ops
+    monkeypatch.setattr(_ops, "SOFTMAX_SLICE_MAX", {torch.float16: (slice_max, slice_max), torch.float32: (slice_max, slice_max)})
+    monkeypatch.setattr(_ops, "SOFTMAX_SLICES", (slices, slices))
+    mask = np.asarray(ZOO["long_row_5x40"])
+    mask = np.concatenate([mask, _tri(40)[:30]], axis=0)
+    y, ref = _fwd(mask, dtype, 0.125, True, batch=(2,), std=2.0, seed=9)
+    assert rel_err(y, ref) <= tol_of(dtype)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    g = torch.Generator().manual_seed(4)
+    yy = torch.rand(2, L.num_blocks, 32, 32, generator=g).to(dtype)
+    dy = torch.randn(2, L.num_blocks, 32, 32, generator=g).to(dtype)
+    dx = sparse_ops.sparse_softmax_backward(yy.cuda(), dy.cuda(), L.row_layout[0], L.row_layout[1], 0.25)
+    assert rel_err(to_np(dx), so.backward(to_np(yy), to_np(dy), mask, 0.25)) <= tol_of(dtype)
