@@ -220,4 +220,27 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
     return check_launch(bsa::launch_softmax_backward(dtype, p, (hipStream_t)stream), "bsa_softmax_backward");
 }
 
+int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out,
+                          const int32_t *row_blocks, const int32_t *row_offsets,
+                          const int32_t *sched, int sched_wgs, int sched_waves,
+                          int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
+                          float scale, int causal, void *stream)
+{
+    const char *who = "bsa_attention_forward";
+    if (dtype != BSA_F16) return fail(BSA_ERR_UNSUPPORTED, "%s: only fp16 (dtype 1) is built, got %d", who, dtype);
+    if (head_dim != 64) return fail(BSA_ERR_UNSUPPORTED, "%s: only head_dim 64 is built, got %d", who, head_dim);
+    if (!q || !k || !v || !out || !row_offsets || (!row_blocks && nnz > 0))
+        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
+    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
+        return fail(BSA_ERR_INVALID, "%s: nnz %d does not fit a %d x %d mask", who, nnz, mask_rows, mask_cols);
+    if (batches < 1) return fail(BSA_ERR_INVALID, "%s: batches %d < 1", who, batches);
+    int rc = check_schedule(sched, sched_wgs, sched_waves, batches, who);
+    if (rc) return rc;
+    bsa::AttentionArgs p{q, k, v, out, row_blocks, sched, mask_rows, sched_wgs, sched_waves,
+                         mask_rows, mask_cols, batches, scale, causal != 0};
+    return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
+}
+
 }  // extern "C"

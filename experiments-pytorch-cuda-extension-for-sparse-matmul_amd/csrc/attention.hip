@@ -1,0 +1,212 @@
+// Fused block-sparse attention forward for gfx950: out = softmax(scale * q k^T, over the stored
+// blocks of a row, causal if asked) v, without the scores ever leaving the chip.
+//
+// The reference computes this as three launches with the scores written and read twice in between
+// (SDD sparse/native/sparse_smm_gpu.cu:22-95, softmax sparse_softmax.cu:113-155, DSD
+// sparse_smm_gpu.cu:106-181, chained by the caller); per stored block that is 2 KB written + 2 KB
+// read + 2 KB written + 2 KB read of HBM traffic that this kernel does not have.
+//
+// One wavefront walks a chunk of the blocks (r, c) of block row r:
+//   S^T = K_c Q_r^T        32 keys x 32 queries, 4 MFMAs over head dim 64; Q_r stays in registers
+//   online softmax          a lane holds ONE query column of S^T (16 keys; the other 16 sit in lane
+//                           l ^ 32), so max, sum and the rescaling factor are per-lane scalars and
+//                           one cross-lane exchange per block
+//   O^T += V_c^T P^T        the probabilities go from the accumulators of the first product straight
+//                           into the operand registers of the second: accumulator value v of lane
+//                           half h is key 8 (v / 4) + 4 h + v % 4, and V_c is parked in LDS with
+//                           its rows exchanged to match (put_strip_swapped_addr).  No LDS round
+//                           trip, no shuffle.
+// The waves of a row (a team of the schedule) merge their (max, sum, O^T) through LDS.
+#include "bsa_device.hpp"
+#include "lds_tiles.hpp"
+#include "bsa_internal.hpp"
+#include "../../include/bsa.h"
+
+namespace bsa {
+
+constexpr int AT_HEAD = 64;                    // head dim
+constexpr int AT_LDS_PER_WAVE = 4096 + 4096 + 512;   // K tile pair + V strip (reused: O^T partial 8 KB) + row stats
+constexpr int AT_DEPTH = 2;
+
+__device__ __forceinline__ float at_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float at_lane_xor32(float x)
+{
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((lane_id() ^ 32) << 2, __float_as_int(x)));
+}
+__device__ __forceinline__ float at_finite_or_zero(float m) { return m == -__builtin_inff() ? 0.f : m; }
+
+__global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
+    const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
+    half_t *__restrict__ out, const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int rows_q, int rows_k, float scale2 /* scale * log2(e) */, int causal)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const bool active = e.group >= 0;
+    const int r = e.group;
+    const int qq = l & 31, h = l >> 5;          // query column of this lane, lane half
+    const float NEG_INF = -__builtin_inff();
+
+    unsigned char *my_lds = lds_raw + (size_t)w * AT_LDS_PER_WAVE;
+    half_t *tile_k = reinterpret_cast<half_t *>(my_lds);            // two [key][32 d] tiles
+    half_t *tile_v = reinterpret_cast<half_t *>(my_lds + 4096);     // [key][64 n] strip, rows exchanged
+    const half_t *kb = k + (size_t)batch * rows_k * AT_HEAD;
+    const half_t *vb = v + (size_t)batch * rows_k * AT_HEAD;
+
+    // Q_r as the column operand of S^T: lane (qq, h) holds d = 16 s + 8 h .. + 7 of query qq
+    h8 qop[AT_HEAD / 16];
+    if (active) {
+        const half_t *qrow = q + ((size_t)batch * rows_q + BS * r + qq) * AT_HEAD + 8 * h;
+#pragma unroll
+        for (int s = 0; s < AT_HEAD / 16; ++s) qop[s] = as_h8(ldg16(qrow + 16 * s));
+    }
+
+    struct Frag { uint4 k0[2], k1[2], vv[4]; };   // K_c as two 32 x 32 tiles (d halves), V_c as a 4 KB strip
+    DescWindow win;
+    auto load = [&](int p, Frag &f) {
+        const int c = win.get(p).col();
+        ldg_tile32(kb + (size_t)(BS * c) * AT_HEAD, AT_HEAD, f.k0);
+        ldg_tile32(kb + (size_t)(BS * c) * AT_HEAD + 32, AT_HEAD, f.k1);
+        const half_t *vs = vb + (size_t)(BS * c) * AT_HEAD;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) f.vv[t] = ldg16(vs + 8 * (l + 64 * t));
+    };
+
+    float m = NEG_INF, lsum = 0.f;               // running max of the query (both lane halves agree), this half's sum
+    f16v oacc[2] = {{0}, {0}};                   // O^T: lane = query column, values = head dims 32 t + 8 (v / 4) + 4 h + v % 4
+
+    auto step = [&](const Frag &f, int c) {
+        wave_lds_fence();
+        lds_put_kc<false>(tile_k, f.k0);
+        lds_put_kc<false>(tile_k + BS2, f.k1);
+        lds_put_strip_swapped(tile_v, f.vv);
+        wave_lds_fence();
+        f16v sacc = {0};
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) sacc = mfma_f16(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
+
+        float sv[16], bm = NEG_INF;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            sv[i] = sacc[i] * scale2;
+            if (causal && c >= r) {
+                const int key = 8 * (i >> 2) + 4 * h + (i & 3);
+                if (c > r || key > qq) sv[i] = NEG_INF;
+            }
+            bm = fmaxf(bm, sv[i]);
+        }
+        bm = fmaxf(bm, at_lane_xor32(bm));
+        const float m_new = fmaxf(m, bm);
+        const float mm = at_finite_or_zero(m_new);
+        const float alpha = at_exp2(m - mm);     // exp2(-inf) = 0: nothing accumulated so far
+        m = m_new;
+        float psum = 0.f;
+        h8 pop[2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float pv = at_exp2(sv[i] - mm);
+            psum += pv;
+            pop[i >> 3][i & 7] = (half_t)pv;
+        }
+        lsum = lsum * alpha + psum;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) oacc[t] = mfma_f16(lds_get_strip<false>(tile_v, 32 * t, s), pop[s], oacc[t]);
+    };
+
+    if (active) {
+        Frag fr[AT_DEPTH];
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+#pragma unroll
+            for (int d = 0; d < AT_DEPTH; ++d)
+                if (seg + d < seg_end) load(seg + d, fr[d]);
+            for (int p = seg; p < seg_end; p += AT_DEPTH) {
+#pragma unroll
+                for (int d = 0; d < AT_DEPTH; ++d) {
+                    if (p + d < seg_end) {
+                        const int c = win.get(p + d).col();
+                        step(fr[d], c);
+                        if (p + d + AT_DEPTH < seg_end) load(p + d + AT_DEPTH, fr[d]);
+                    }
+                }
+            }
+        }
+    }
+    lsum += at_lane_xor32(lsum);                 // both halves used the same max
+
+    // team merge: every wave but the leader parks (max, sum, O^T); the leader rescales and adds
+    const int slot0 = e.first_wave(), nw = e.team_waves();
+    const bool leader = active && w == slot0;
+    float *park = reinterpret_cast<float *>(my_lds);                  // 2048 floats of O^T
+    float2 *stat = reinterpret_cast<float2 *>(my_lds + 8192);         // 32 (max, sum)
+    if (active && !leader) {
+        wave_lds_fence();
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) park[(t * 16 + i) * WAVE + l] = oacc[t][i];
+        if (h == 0) stat[qq] = make_float2(m, lsum);
+    }
+    __syncthreads();
+    if (!leader) return;
+    if (nw > 1) {
+        float M = m;
+        for (int o = 1; o < nw; ++o)
+            M = fmaxf(M, reinterpret_cast<const float2 *>(lds_raw + (size_t)(w + o) * AT_LDS_PER_WAVE + 8192)[qq].x);
+        const float MM = at_finite_or_zero(M);
+        const float mine = at_exp2(m - MM);
+        lsum *= mine;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[t][i] *= mine;
+        for (int o = 1; o < nw; ++o) {
+            const unsigned char *other = lds_raw + (size_t)(w + o) * AT_LDS_PER_WAVE;
+            const float2 st = reinterpret_cast<const float2 *>(other + 8192)[qq];
+            const float f = at_exp2(st.x - MM);
+            lsum += st.y * f;
+            const float *op = reinterpret_cast<const float *>(other);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[t][i] += op[(t * 16 + i) * WAVE + l] * f;
+        }
+    }
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+    half_t *orow = out + ((size_t)batch * rows_q + BS * r + qq) * AT_HEAD + 4 * h;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            h4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (half_t)(oacc[t][4 * g + j] * inv);
+            *reinterpret_cast<h4 *>(orow + 32 * t + 8 * g) = o;
+        }
+    }
+}
+
+hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t st)
+{
+    dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
+    attention_fwd_f16_kernel<<<grid, block, (size_t)p.sched_waves * AT_LDS_PER_WAVE, st>>>(
+        (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (half_t *)p.out,
+        (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches,
+        32 * p.mask_rows, 32 * p.mask_cols, p.scale * 1.4426950408889634f, p.causal ? 1 : 0);
+    return hipGetLastError();
+}
+
+}  // namespace bsa

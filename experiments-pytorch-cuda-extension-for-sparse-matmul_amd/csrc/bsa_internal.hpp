@@ -50,4 +50,18 @@ struct SoftmaxArgs {
 hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t stream);
 hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t stream);
 
+struct AttentionArgs {
+    const void *q, *k, *v;
+    void *out;
+    const int32_t *blocks;
+    const int32_t *sched;
+    int groups;
+    int sched_wgs, sched_waves;
+    int mask_rows, mask_cols, batches;
+    float scale;
+    bool causal;
+};
+
+hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t stream);
+
 }  // namespace bsa

@@ -80,6 +80,17 @@ BSA_HD constexpr int put_strip_addr(int lane, int q)
     int k = c >> 3;
     return 16 * (k * 8 + ((c & 7) ^ strip_swizzle(k)));
 }
+// The same strip with rows 4-7 and 8-11 of every 16 exchanged (bits 2 and 3 of k): a reader
+// that asks for row 16 s + 8 h + j then gets row 16 s + 8 (j / 4) + 4 h + j % 4, the row an MFMA
+// accumulator lane (h = lane / 32) holds as its value 8 s + j.  The fused attention kernel feeds its
+// probabilities to the second product straight out of the first one's accumulators this way.
+BSA_HD constexpr int swap_bits23(int k) { return (k & ~12) | ((k & 4) << 1) | ((k & 8) >> 1); }
+BSA_HD constexpr int put_strip_swapped_addr(int lane, int q)
+{
+    int c = lane + 64 * q;
+    int k = swap_bits23(c >> 3);
+    return 16 * (k * 8 + ((c & 7) ^ strip_swizzle(k)));
+}
 BSA_HD constexpr int get_strip_addr(bool permuted, int lane, int step, int half, int x0)
 {
     int g = lane >> 4, s = lane & 15;

@@ -84,6 +84,15 @@ __device__ __forceinline__ void lds_put_strip(half_t *tile, const uint4 (&lo)[2]
         *reinterpret_cast<uint4 *>(lds_bytes(tile) + put_strip_addr(l, q)) = q < 2 ? lo[q & 1] : hi[q & 1];
 }
 
+// rows 4-7 and 8-11 of every 16 exchanged (see put_strip_swapped_addr)
+__device__ __forceinline__ void lds_put_strip_swapped(half_t *tile, const uint4 (&raw)[4])
+{
+    int l = lane_id();
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<uint4 *>(lds_bytes(tile) + put_strip_swapped_addr(l, q)) = raw[q];
+}
+
 template <bool PERMUTED>
 __device__ __forceinline__ h8 lds_get_strip(const half_t *tile, int x0, int step)
 {

@@ -1,5 +1,6 @@
 from .layout import SparseLayout
 from .matmul import matmul
 from .softmax import softmax
+from .attention import attention
 
-__all__ = ["SparseLayout", "matmul", "softmax"]
+__all__ = ["SparseLayout", "matmul", "softmax", "attention"]

@@ -16,6 +16,7 @@ SCHEDULE_GROUP_WALK_LONG = (8, 4)    # tables with longer groups (columns of cau
 GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
+SCHEDULE_ATTENTION = (8, 4)           # fused forward: rows are never split across workgroups
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
@@ -223,3 +224,43 @@ def sparse_softmax_backward(y, dy, row_blocks, row_table, scale=1.0, col_layout=
             row_table.data_ptr(), sched.table.data_ptr(), sched.workgroups, sched.waves,
             mask_rows, mask_cols, nnz, batches, float(scale), _k.current_stream()))
     return dx
+
+
+def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=False, col_layout=None):
+    """``softmax(scale * q k^T on the stored blocks) v`` in one launch: the chain of
+    ``sparse_matmul('sdd', trans_b)``, the softmax and ``sparse_matmul('dsd')`` (sparse/matmul.py:57,
+    sparse_softmax.cu:208-231) without the scores in memory.  fp16, head dim 64."""
+    row_layout = (row_blocks, row_table)
+    _check_layout(row_layout, "row_layout")
+    for t, name in ((q, "q"), (k, "k"), (v, "v")):
+        if t.dtype != torch.float16:
+            raise TypeError(f"{name} must be float16, got {t.dtype}")
+        if not t.is_cuda or t.device != q.device:
+            raise ValueError("q, k, v must live on the same GPU")
+        if t.dim() < 3:
+            raise ValueError(f"{name} needs at least one batch dimension, got shape {tuple(t.shape)}")
+    if row_blocks.device != q.device:
+        raise ValueError("layout tables and operands must live on the same GPU")
+    mask_rows = row_table.numel() - 1
+    if col_layout is None:
+        raise ValueError("col_layout is needed for the number of block columns")
+    mask_cols = col_layout[1].numel() - 1
+    nnz = row_blocks.numel() // 2
+    head = q.size(-1)
+    if q.size(-2) != mask_rows * BLOCK or k.size(-2) != mask_cols * BLOCK or k.shape != v.shape \
+            or k.size(-1) != head or q.shape[:-2] != k.shape[:-2]:
+        raise ValueError(f"q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit a "
+                         f"{mask_rows} x {mask_cols} block layout")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    out = torch.empty_like(q)
+    if out.numel() == 0:
+        return out
+    batches = q.numel() // (q.size(-1) * q.size(-2))
+    cap, waves = SCHEDULE_ATTENTION
+    sched = schedule_for(row_layout, (cap, waves, False))
+    with torch.cuda.device(q.device):
+        _k.check(_k.lib.bsa_attention_forward(
+            _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+            row_blocks.data_ptr(), row_table.data_ptr(), sched.table.data_ptr(), sched.workgroups, sched.waves,
+            mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), _k.current_stream()))
+    return out

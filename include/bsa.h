@@ -163,6 +163,25 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
                          int mask_rows, int mask_cols, int nnz, int batches,
                          float scale, void *stream);
 
+/* ---- fused block-sparse attention, forward ----------------------------------
+ * out = softmax_row(scale * q k^T restricted to the stored blocks, causal if asked) v in one launch:
+ * the chain SDD -> softmax -> DSD that a caller of the reference writes with two calls of
+ * sparse_matmul (sparse/matmul.py:57, kernels sparse_smm_gpu.cu:22-95 and :106-181) around the
+ * softmax of sparse_softmax.cu:113-155, without the [batches, nnz, 32, 32] scores ever being
+ * stored.  Same meaning as bsa_matmul(SDD, q, k, tr_b = 1), bsa_softmax_forward, bsa_matmul(DSD)
+ * in a row; the probabilities are rounded to fp16 before the second product, as there.
+ *   q    [batches, 32 * mask_rows, head_dim], k, v  [batches, 32 * mask_cols, head_dim], contiguous
+ *   out  [batches, 32 * mask_rows, head_dim]; rows without stored (or unmasked) blocks give zeros
+ *   tables / schedule: those of the ROW layout; the schedule must be built with
+ *   allow_split = 0 and slice_max = -1 (a block row stays inside one workgroup).
+ * fp16 only (BSA_ERR_UNSUPPORTED otherwise), head_dim 64.
+ */
+int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out,
+                          const int32_t *row_blocks, const int32_t *row_offsets,
+                          const int32_t *sched, int sched_wgs, int sched_waves,
+                          int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
+                          float scale, int causal, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,111 @@
+"""GPU: fused block-sparse attention against the float64 oracle and against the unfused chain."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention_oracle as ao
+from helpers import mask_zoo, rel_err, to_np
+
+pytestmark = pytest.mark.gpu
+ZOO = dict(mask_zoo())
+TOL = 2e-3          # fp16 operands, fp32 accumulation, probabilities rounded to fp16 (as in the chain)
+
+
+def _qkv(mask, batch=(2,), seed=0, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    r, c = np.asarray(mask).shape
+    mk = lambda n: (std * torch.randn(*batch, 32 * n, 64, generator=g)).half()
+    return mk(r), mk(c), mk(c)
+
+
+def _run(mask, scale, causal, **kw):
+    import sparse
+    q, k, v = _qkv(mask, **kw)
+    L = sparse.SparseLayout(torch.as_tensor(np.asarray(mask)))
+    out = sparse.attention(q.cuda(), k.cuda(), v.cuda(), L, scale, causal)
+    assert out.dtype == torch.float16 and out.shape == q.shape
+    return to_np(out), ao.forward(to_np(q), to_np(k), to_np(v), mask, scale, causal)
+
+
+@pytest.mark.parametrize("scale,causal", [(0.125, False), (0.125, True), (1.0, False), (1.0, True)])
+@pytest.mark.parametrize("name", ["known3x3", "single", "one_cell", "full4", "empty_row_col_6x5",
+                                  "wide_2x9", "rand16", "long_row_5x40", "long_col_70x3"])
+def test_forward(name, scale, causal):
+    out, ref = _run(np.asarray(ZOO[name]), scale, causal)
+    assert np.all(np.isfinite(out))
+    assert rel_err(out, ref) <= TOL
+
+
+def test_rows_that_see_nothing_give_zeros():
+    mask = np.array([[0, 1], [1, 1], [0, 0]])
+    out, ref = _run(mask, 1.0, True)
+    assert np.all(out[:, :32] == 0) and np.all(out[:, 64:] == 0)       # block (0, 1) is right of the diagonal
+    assert rel_err(out, ref) <= TOL
+
+
+def test_long_rows_and_multi_dim_batch():
+    mask = np.zeros((3, 256), dtype=np.int64)
+    mask[0, :] = 1
+    mask[1, ::5] = 1
+    mask[2, 200:] = 1
+    out, ref = _run(mask, 0.125, False, batch=(2, 2), seed=4)
+    assert rel_err(out, ref) <= TOL
+
+
+def test_large_logits_stay_finite():
+    out, ref = _run(np.asarray(ZOO["known3x3"]), 1.0, False, std=6.0, seed=2)   # logits of +-300
+    assert np.all(np.isfinite(out)) and rel_err(out, ref) <= TOL
+
+
+def test_matches_the_unfused_chain_on_config5():
+    import sparse, workloads as wl
+    cfg = wl.config5()
+    L = sparse.SparseLayout(cfg["mask"])
+    q, k, v = (cfg[n].cuda() for n in ("q", "k", "v"))
+    fused = sparse.attention(q, k, v, L, cfg["scale"], cfg["causal"])
+    s = sparse.matmul(q, k, "sdd", L, False, True)
+    p = sparse.softmax(s, L, cfg["scale"], cfg["causal"])
+    chain = sparse.matmul(p, v, "dsd", L)
+    err = ((fused.float() - chain.float()).abs().max() / chain.float().abs().max()).item()
+    assert err <= 2e-3
+    b, h = 1, 5
+    ref = ao.forward(to_np(cfg["q"][b, h][None]), to_np(cfg["k"][b, h][None]), to_np(cfg["v"][b, h][None]),
+                     cfg["mask"].numpy(), cfg["scale"], cfg["causal"])
+    assert rel_err(to_np(fused[b, h][None]), ref) <= TOL
+
+
+def test_gradients_match_the_unfused_chain():
+    import sparse
+    mask = np.asarray(ZOO["rand16"])
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    q, k, v = (t.cuda().requires_grad_(True) for t in _qkv(mask, seed=7))
+    g = torch.randn(q.shape, generator=torch.Generator().manual_seed(8)).half().cuda()
+    sparse.attention(q, k, v, L, 0.125, True).backward(g)
+    got = [t.grad.clone() for t in (q, k, v)]
+    for t in (q, k, v):
+        t.grad = None
+    s = sparse.matmul(q, k, "sdd", L, False, True)
+    o = sparse.matmul(sparse.softmax(s, L, 0.125, True), v, "dsd", L)
+    o.backward(g)
+    for a, t in zip(got, (q, k, v)):
+        assert rel_err(to_np(a), to_np(t.grad)) <= 2e-3
+    # and against float64 autograd of the dense meaning
+    qd, kd, vd = (t.detach().double().cpu().requires_grad_(True) for t in (q, k, v))
+    vis = torch.as_tensor(mask).bool().repeat_interleave(32, 0).repeat_interleave(32, 1) & torch.ones(512, 512).tril().bool()
+    sc = (0.125 * qd @ kd.transpose(-1, -2)).masked_fill(~vis, float("-inf"))
+    (torch.softmax(sc, -1) @ vd).backward(g.double().cpu())
+    for a, t in zip(got, (qd, kd, vd)):
+        assert rel_err(to_np(a), t.grad.numpy()) <= 4e-3
+
+
+def test_argument_checks():
+    import sparse
+    mask = np.asarray(ZOO["known3x3"])
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    q, k, v = (t.cuda() for t in _qkv(mask))
+    with pytest.raises(TypeError):
+        sparse.attention(q.float(), k.float(), v.float(), L)
+    with pytest.raises(ValueError):
+        sparse.attention(q[:, :64], k, v, L)
+    with pytest.raises(Exception):
+        sparse.attention(q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous(), L)
