@@ -9,7 +9,8 @@ A step is one pass of the three products over that batch:
     DDS  grad   = dy^T @ w  -> [16, 64, 4096]         (reads 1530 blocks/head, dy)
 
 `value` = nnz-block TFLOP/s = 3 * 2 * nnz * 32 * 32 * 64 * 16 flop / step time.
-The softmax (scale 1/8, causal) is timed in its own loop and reported in GB/s.
+The softmax (scale 1/8, causal) is timed in its own loop and reported in GB/s, and the
+attention forward q, k, v -> out as one fused launch next to the chain of three.
 Consecutive launches take the next of several resident operand sets, so every
 launch finds its operands in HBM, not in the 256 MB infinity cache (`--sets 1`
 shows the cache-resident figures).  Launches are replayed
@@ -154,6 +155,26 @@ def main():
             per_op[name]["nnz_TFLOPs"] = round(tf, 2)
             per_op[name]["mfma_frac"] = round(tf / MFMA_F16_PEAK_TFLOPS, 4)
 
+    # attention forward as a whole, q k v -> out: one fused launch against the chain of three launches
+    # (the two products of a forward pass are 2 * flops_one); not part of `value`
+    def chain(w):
+        s = sparse.matmul(w["q"], w["k"], "sdd", layout, False, True)
+        return sparse.matmul(sparse.softmax(s, layout, 0.125, True), w["v"], "dsd", layout)
+
+    def fused(w):
+        return sparse.attention(w["q"], w["k"], w["v"], layout, 0.125, True)
+
+    with torch.no_grad():
+        a, b = fused(sets[0]), chain(sets[0])
+        err = ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+        assert err <= 2e-3, f"fused attention differs from the chain: {err}"
+    attention = {}
+    for name, fn in (("fused", fused), ("chain", chain)):
+        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+        attention[name + "_us"] = round(ms * 1e3, 3)
+        attention[name + "_nnz_TFLOPs"] = round(2 * flops_one / (ms * 1e-3) / 1e12, 2)
+    attention["speedup"] = round(attention["chain_us"] / attention["fused_us"], 2)
+
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/): same
     # workload, same kernels; absent file -> null
     traffic = {}
@@ -182,6 +203,7 @@ def main():
                                  "unit": "GB/s", "frac": per_op["softmax"]["hbm_frac"],
                                  "traffic": traffic.get("softmax")}},
         "kernels": per_op,
+        "attention_forward": attention,
     }
 
     if not args.no_cpu:

@@ -24,9 +24,15 @@
 
 namespace bsa {
 
+#ifdef BSA_AT_ABLATE   // debug builds: 1 no softmax math, 2 no S product, 4 no PV product, 8 no staging, 16 loads once
+#define AT_ABLATE(bit) ((BSA_AT_ABLATE) & (bit))
+#else
+#define AT_ABLATE(bit) 0
+#endif
+
 constexpr int AT_HEAD = 64;                    // head dim
 constexpr int AT_LDS_PER_WAVE = 4096 + 4096 + 512;   // K tile pair + V strip (reused: O^T partial 8 KB) + row stats
-constexpr int AT_DEPTH = 2;
+constexpr float AT_LAZY = 8.f;                // log2 of the growth of a row maximum that forces a rescale
 
 __device__ __forceinline__ float at_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float at_lane_xor32(float x)
@@ -79,69 +85,105 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     float m = NEG_INF, lsum = 0.f;               // running max of the query (both lane halves agree), this half's sum
     f16v oacc[2] = {{0}, {0}};                   // O^T: lane = query column, values = head dims 32 t + 8 (v / 4) + 4 h + v % 4
 
-    auto step = [&](const Frag &f, int c) {
+    // registers -> staging tiles; the registers are free for the next block's loads afterwards
+    auto stage = [&](const Frag &f) {
+        if (AT_ABLATE(8)) return;
         wave_lds_fence();
         lds_put_kc<false>(tile_k, f.k0);
         lds_put_kc<false>(tile_k + BS2, f.k1);
         lds_put_strip_swapped(tile_v, f.vv);
         wave_lds_fence();
+    };
+    auto step = [&](int c) {
         f16v sacc = {0};
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-            for (int s = 0; s < 2; ++s) sacc = mfma_f16(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
-
-        float sv[16], bm = NEG_INF;
+            for (int s = 0; s < 2; ++s)
+                if (!AT_ABLATE(2)) sacc = mfma_f16(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
+        if (AT_ABLATE(1)) {
+            h8 pq[2];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            sv[i] = sacc[i] * scale2;
-            if (causal && c >= r) {
+            for (int i = 0; i < 16; ++i) pq[i >> 3][i & 7] = (half_t)sacc[i];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (!AT_ABLATE(4)) oacc[t] = mfma_f16(lds_get_strip<false>(tile_v, 32 * t, s), pq[s], oacc[t]);
+            return;
+        }
+
+        // Row maximum of the scaled scores.  Off the diagonal nothing is masked and the scale is
+        // folded into the exponent (one fused multiply-add per score); the diagonal block of a
+        // causal launch takes the explicit route.
+        float bm;
+        const bool masked = causal && c >= r;
+        float mul = scale2;                      // what is still to be applied to sacc in the exponent
+        if (masked) {
+            bm = NEG_INF;
+            mul = 1.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
                 const int key = 8 * (i >> 2) + 4 * h + (i & 3);
-                if (c > r || key > qq) sv[i] = NEG_INF;
+                sacc[i] = (c > r || key > qq) ? NEG_INF : sacc[i] * scale2;
+                bm = fmaxf(bm, sacc[i]);
             }
-            bm = fmaxf(bm, sv[i]);
+        } else {
+            float hi = sacc[0], lo = sacc[0];
+#pragma unroll
+            for (int i = 1; i < 16; ++i) {
+                hi = fmaxf(hi, sacc[i]);
+                if (scale2 < 0.f) lo = fminf(lo, sacc[i]);     // uniform: a negative scale turns the order round
+            }
+            bm = scale2 < 0.f ? lo * scale2 : hi * scale2;
         }
         bm = fmaxf(bm, at_lane_xor32(bm));
-        const float m_new = fmaxf(m, bm);
-        const float mm = at_finite_or_zero(m_new);
-        const float alpha = at_exp2(m - mm);     // exp2(-inf) = 0: nothing accumulated so far
-        m = m_new;
+        // Lazy rescaling: the reference point m only moves when some row's maximum has grown by
+        // more than 2^AT_LAZY since it was set, so the 32 multiplies of O^T (and the branch is
+        // uniform) are skipped for most blocks; until then probabilities may reach 2^AT_LAZY,
+        // which fp16 holds without loss of relative precision.
+        if (__builtin_amdgcn_ballot_w64(bm > m + AT_LAZY) != 0ull) {
+            const float m_new = fmaxf(m, bm);
+            const float alpha = at_exp2(at_finite_or_zero(m) - at_finite_or_zero(m_new));
+            const float keep = m == NEG_INF ? 0.f : alpha;      // nothing accumulated so far
+            m = m_new;
+            lsum *= keep;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[t][i] *= keep;
+        }
+        const float mm = at_finite_or_zero(m);
         float psum = 0.f;
         h8 pop[2];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float pv = at_exp2(sv[i] - mm);
+            const float pv = at_exp2(__builtin_fmaf(sacc[i], mul, -mm));
             psum += pv;
             pop[i >> 3][i & 7] = (half_t)pv;
         }
-        lsum = lsum * alpha + psum;
+        lsum += psum;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int s = 0; s < 2; ++s) oacc[t] = mfma_f16(lds_get_strip<false>(tile_v, 32 * t, s), pop[s], oacc[t]);
+            for (int s = 0; s < 2; ++s)
+                if (!AT_ABLATE(4)) oacc[t] = mfma_f16(lds_get_strip<false>(tile_v, 32 * t, s), pop[s], oacc[t]);
+                else oacc[t][s] += (float)pop[s][0];
     };
 
+    // One block in flight: its tiles are requested as soon as the previous block's have been copied
+    // to LDS, so the loads run under the previous block's products and softmax.  (A second set of
+    // load registers costs an occupancy step, which measured worse than the shorter prefetch.)
     if (active) {
-        Frag fr[AT_DEPTH];
+        Frag fr;
         for (int seg = e.begin; seg < e.end; seg += WAVE) {
             const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
             win.fetch(blocks, seg, seg_end);
-#pragma unroll
-            for (int d = 0; d < AT_DEPTH; ++d)
-                if (seg + d < seg_end) load(seg + d, fr[d]);
-            for (int p = seg; p < seg_end; p += AT_DEPTH) {
-#pragma unroll
-                for (int d = 0; d < AT_DEPTH; ++d) {
-                    if (p + d < seg_end) {
-                        const int c = win.get(p + d).col();
-                        step(fr[d], c);
-                        if (p + d + AT_DEPTH < seg_end) load(p + d + AT_DEPTH, fr[d]);
-                    }
-                }
+            load(seg, fr);
+            for (int p = seg; p < seg_end; ++p) {
+                stage(fr);
+                if (p + 1 < seg_end && !AT_ABLATE(16)) load(p + 1, fr);
+                step(win.get(p).col());
             }
         }
     }

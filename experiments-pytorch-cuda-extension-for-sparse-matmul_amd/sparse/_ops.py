@@ -16,7 +16,7 @@ SCHEDULE_GROUP_WALK_LONG = (8, 4)    # tables with longer groups (columns of cau
 GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
-SCHEDULE_ATTENTION = (8, 4)           # fused forward: rows are never split across workgroups
+SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
