@@ -61,6 +61,17 @@ __global__ __launch_bounds__(256) void probe(const int *offs, unsigned long long
             for (int u = 0; u < 16; ++u) asm volatile("ds_write_b128 %0, %1" ::"v"(addr), "v"(w) : "memory");
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             acc += 1;
+        } else if (WIDTH == -64) {   // ds_write_b64
+            u2 w = {acc, acc + 1};
+#pragma unroll
+            for (int u = 0; u < 16; ++u) asm volatile("ds_write_b64 %0, %1" ::"v"(addr), "v"(w) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            acc += 1;
+        } else if (WIDTH == -32) {   // ds_write_b32
+#pragma unroll
+            for (int u = 0; u < 16; ++u) asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(acc) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            acc += 1;
         } else {                     // ds_read_b64_tr_b16
             u2 v[16];
 #pragma unroll
@@ -102,14 +113,16 @@ static std::vector<int> pattern(int (*f)(int))
 }
 
 // `./lds_bank_probe OP a0,a1,...,a63 [label]` times one caller-supplied pattern (byte offsets per
-// lane); OP is b128, b64, b32 (reads), w128 (ds_write_b128) or tr64 (ds_read_b64_tr_b16).
+// lane); OP is b128, b64, b32 (reads), w128, w64, w32 (ds_write_b128 / _b64 / _b32) or tr64
+// (ds_read_b64_tr_b16).
 static int custom(int argc, char **argv)
 {
     std::vector<int> v;
     for (char *tok = strtok(argv[2], ","); tok; tok = strtok(nullptr, ",")) v.push_back(atoi(tok));
     if (v.size() != 64) { printf("need 64 offsets\n"); return 1; }
     double t = !strcmp(argv[1], "b128") ? run<16>(v) : !strcmp(argv[1], "b64") ? run<8>(v)
-             : !strcmp(argv[1], "w128") ? run<-16>(v) : !strcmp(argv[1], "tr64") ? run<-8>(v) : run<4>(v);
+             : !strcmp(argv[1], "w128") ? run<-16>(v) : !strcmp(argv[1], "w64") ? run<-64>(v)
+             : !strcmp(argv[1], "w32") ? run<-32>(v) : !strcmp(argv[1], "tr64") ? run<-8>(v) : run<4>(v);
     printf("%s %7.2f\n", argc > 3 ? argv[3] : "custom", t);
     return 0;
 }
@@ -144,5 +157,9 @@ int main(int argc, char **argv)
         {"stride128", [](int l) { return 128 * l; }},
     };
     for (const P &p : b32) printf("b32  %-40s %7.2f\n", p.name, run<4>(pattern(p.f)));
+    printf("w128 %-40s %7.2f\n", "linear", run<-16>(pattern([](int l) { return 16 * l; })));
+    printf("w64  %-40s %7.2f\n", "linear", run<-64>(pattern([](int l) { return 8 * l; })));
+    printf("w64  %-40s %7.2f\n", "stride16 (half of a b128 pattern)", run<-64>(pattern([](int l) { return 16 * l; })));
+    printf("w32  %-40s %7.2f\n", "linear", run<-32>(pattern([](int l) { return 4 * l; })));
     return 0;
 }
