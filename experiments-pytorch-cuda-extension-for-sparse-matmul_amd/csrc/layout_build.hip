@@ -131,15 +131,18 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
     const int tid = (int)threadIdx.x;
     int4 *meta = sched;
     int4 *slots = sched + groups;
-    // Serial first-fit.  Row-sliced groups come first and fill whole workgroups of their own (their
-    // waves need no barrier); then the others: a team (the waves of one part) never straddles a
-    // workgroup boundary.
+    // Serial first-fit in three passes.  Row-sliced groups come first and fill whole workgroups of
+    // their own (their waves need no barrier).  Split groups come next: their parts meet in a
+    // workspace after the walk, and workgroups are dispatched in slot order, so starting them first
+    // lets that exchange run while the rest of the launch is still multiplying.  Then the others.
+    // A team (the waves of one part) never straddles a workgroup boundary.
     if (tid == 0) {
         int pos = 0, tile_slots = 0, split_groups = 0;
-        for (int pass = 0; pass < 2; ++pass) {
+        for (int pass = 0; pass < 3; ++pass) {
             for (int g = 0; g < groups; ++g) {
                 const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split, slice_max, slices);
-                if (gp.sliced != (pass == 0)) continue;
+                const int cls = gp.sliced ? 0 : (gp.parts > 1 ? 1 : 2);
+                if (cls != pass) continue;
                 if (gp.sliced) {
                     meta[g] = make_int4(pos, -1, -1, gp.parts);
                     pos += gp.parts;
