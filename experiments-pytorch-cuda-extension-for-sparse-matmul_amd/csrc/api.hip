@@ -74,6 +74,41 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
                         "bsa_layout_build");
 }
 
+static int check_block_copy(const char *who, int dtype, const void *a, const void *b, const void *t0, const void *t1,
+                            int mask_rows, int mask_cols, int nnz, int batches)
+{
+    if (dtype != BSA_F32 && dtype != BSA_F16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: unsupported dtype %d (fp32 = 0, fp16 = 1)", who, dtype);
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
+    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
+        return fail(BSA_ERR_INVALID, "%s: nnz %d does not fit a %d x %d mask", who, nnz, mask_rows, mask_cols);
+    if (batches < 1) return fail(BSA_ERR_INVALID, "%s: batches %d < 1", who, batches);
+    if (!a || !t0 || !t1 || (!b && nnz > 0)) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    return BSA_OK;
+}
+
+int bsa_to_sparse(int dtype, const void *dense, void *sparse, const int32_t *row_blocks,
+                  int mask_rows, int mask_cols, int nnz, int batches, void *stream)
+{
+    if (nnz == 0 && dense) return BSA_OK;
+    int rc = check_block_copy("bsa_to_sparse", dtype, dense, sparse, row_blocks, row_blocks, mask_rows, mask_cols, nnz, batches);
+    if (rc) return rc;
+    return check_launch(bsa::launch_to_sparse(dtype == BSA_F16 ? 2 : 4, dense, sparse, row_blocks, nnz, batches,
+                                              mask_rows, mask_cols, (hipStream_t)stream), "bsa_to_sparse");
+}
+
+int bsa_to_dense(int dtype, const void *sparse, void *dense, const uint8_t *mask, const int32_t *ordinals,
+                 int mask_rows, int mask_cols, int nnz, int batches, void *stream)
+{
+    int rc = check_block_copy("bsa_to_dense", dtype, dense, sparse, mask, ordinals, mask_rows, mask_cols, nnz, batches);
+    if (rc) return rc;
+    if ((long long)mask_rows * mask_cols > (1LL << 31) - 8)
+        return fail(BSA_ERR_INVALID, "bsa_to_dense: %d x %d cells do not fit the launch", mask_rows, mask_cols);
+    return check_launch(bsa::launch_to_dense(dtype == BSA_F16 ? 2 : 4, sparse, dense, mask, ordinals, nnz, batches,
+                                             mask_rows, mask_cols, (hipStream_t)stream), "bsa_to_dense");
+}
+
 int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves)
 {
     if (groups < 1 || nnz < 0 || cap < 1 || waves < 1) return 0;

@@ -14,6 +14,11 @@ hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, in
                                  int allow_split, int slice_max, int slices, int32_t *sched, int64_t capacity,
                                  int32_t *counts_out, hipStream_t stream);
 
+hipError_t launch_to_sparse(int elem_size, const void *dense, void *sparse, const int32_t *row_blocks,
+                            int nnz, int batches, int R, int C, hipStream_t stream);
+hipError_t launch_to_dense(int elem_size, const void *sparse, void *dense, const uint8_t *mask,
+                           const int32_t *ordinal_of, int nnz, int batches, int R, int C, hipStream_t stream);
+
 struct MatmulArgs {
     const void *a, *b;
     void *c;

@@ -3,10 +3,12 @@
 Same class, attributes and methods as ``sparse/layout.py:5-57`` of the
 reference.  What changed underneath: the two tables are built by one device
 kernel from the uploaded mask (``bsa_layout_build``) instead of CPU torch ops
-and four host-to-device copies; ``to_sparse`` / ``to_dense`` are single gathers
-instead of Python loops over the blocks; ``to_dense`` fills absent blocks with
-zeros (the reference leaves them uninitialised); a bool mask means the same as
-the 0/1 integer mask.
+and four host-to-device copies; ``to_sparse`` / ``to_dense`` of fp16 / fp32 tensors
+on the GPU are one copy kernel each (``bsa_to_sparse`` / ``bsa_to_dense``) instead
+of Python loops over the blocks, differentiable, and ``to_dense`` fills absent
+blocks with zeros (the reference leaves them uninitialised); other tensors (host
+memory, other dtypes) take a torch gather; a bool mask means the same as the 0/1
+integer mask.
 """
 from typing import Tuple
 
@@ -15,6 +17,21 @@ import torch
 from . import kernel as _k
 
 BLOCK = 32
+_COPY_DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
+
+
+class _BlockCopy(torch.autograd.Function):
+    """to_sparse (gather = True) / to_dense through the copy kernels; each is the other's gradient."""
+
+    @staticmethod
+    def forward(ctx, x, layout, gather):
+        ctx.layout, ctx.gather = layout, gather
+        return layout._copy_blocks(x, gather)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return ctx.layout._copy_blocks(grad, not ctx.gather), None, None
+
 
 
 class SparseLayout:
@@ -45,6 +62,8 @@ class SparseLayout:
                 workspace.data_ptr(), _k.current_stream()))
         nnz = int(nnz_dev.item())
         self.num_blocks = nnz
+        self._mask = mask
+        self._ordinals = workspace          # int32[rows * cols]: block index of every stored cell
         # exact-size tensors: the boundary derives nnz from blocks.size(0) / 2 (sparse_kernels.cc:13)
         self.row_layout: Tuple[torch.Tensor, torch.Tensor] = (row_blocks[:2 * nnz].clone(), row_offsets)
         self.col_layout: Tuple[torch.Tensor, torch.Tensor] = (col_blocks[:2 * nnz].clone(), col_offsets)
@@ -59,11 +78,38 @@ class SparseLayout:
             return self._cell_index.to(device)
         return self._cell_index
 
+    def _on_device_path(self, x: torch.Tensor) -> bool:
+        return x.is_cuda and x.device == self.device and x.dtype in _COPY_DTYPES
+
+    def _copy_blocks(self, x: torch.Tensor, gather: bool) -> torch.Tensor:
+        rows, cols = self.pattern.shape
+        x = x.contiguous()
+        lead = x.shape[:-2] if gather else x.shape[:-3]
+        shape = lead + ((self.num_blocks, BLOCK, BLOCK) if gather else (rows * BLOCK, cols * BLOCK))
+        out = torch.empty(shape, dtype=x.dtype, device=x.device)
+        batches = 1
+        for n in lead:
+            batches *= n
+        if out.numel() == 0 or batches == 0:
+            return out
+        with torch.cuda.device(self.device):
+            if gather:
+                _k.check(_k.lib.bsa_to_sparse(_COPY_DTYPES[x.dtype], x.data_ptr(), out.data_ptr(),
+                                              self.row_layout[0].data_ptr(), rows, cols, self.num_blocks, batches,
+                                              _k.current_stream()))
+            else:
+                _k.check(_k.lib.bsa_to_dense(_COPY_DTYPES[x.dtype], x.data_ptr(), out.data_ptr(),
+                                             self._mask.data_ptr(), self._ordinals.data_ptr(), rows, cols,
+                                             self.num_blocks, batches, _k.current_stream()))
+        return out
+
     def to_sparse(self, x: torch.Tensor) -> torch.Tensor:
         """``[..., R*32, C*32]`` -> ``[..., nnz, 32, 32]`` (layout.py:40-45)."""
         rows, cols = self.pattern.shape
         if tuple(x.shape[-2:]) != (rows * BLOCK, cols * BLOCK):
             raise ValueError(f"expected [..., {rows * BLOCK}, {cols * BLOCK}], got {tuple(x.shape)}")
+        if self._on_device_path(x):
+            return _BlockCopy.apply(x, self, True)
         tiles = x.reshape(x.shape[:-2] + (rows, BLOCK, cols, BLOCK)).transpose(-3, -2)
         tiles = tiles.reshape(x.shape[:-2] + (rows * cols, BLOCK, BLOCK))
         return tiles.index_select(-3, self._index_on(x.device)).contiguous()
@@ -73,6 +119,8 @@ class SparseLayout:
         rows, cols = self.pattern.shape
         if tuple(x.shape[-3:]) != (self.num_blocks, BLOCK, BLOCK):
             raise ValueError(f"expected [..., {self.num_blocks}, 32, 32], got {tuple(x.shape)}")
+        if self._on_device_path(x):
+            return _BlockCopy.apply(x, self, False)
         tiles = x.new_zeros(x.shape[:-3] + (rows * cols, BLOCK, BLOCK))
         tiles.index_copy_(-3, self._index_on(x.device), x)
         tiles = tiles.reshape(x.shape[:-3] + (rows, cols, BLOCK, BLOCK)).transpose(-3, -2)

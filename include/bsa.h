@@ -69,7 +69,10 @@ const char *bsa_last_error(void);
  *   col_blocks   device int32[2*R*C]
  *   col_offsets  device int32[C+1]
  *   nnz_out      device int32[1]
- *   workspace    device, bsa_layout_workspace_bytes(R, C) bytes
+ *   workspace    device, bsa_layout_workspace_bytes(R, C) bytes; afterwards it holds, as
+ *                int32[R*C], for every cell the number of stored blocks in front of
+ *                it in row-major order (the block index of a stored cell), which
+ *                bsa_to_dense reads
  * Limits: 1 <= R <= 32767, 1 <= C <= 65535 (the packed position is 16+16 bit
  * in a signed int32).
  */
@@ -78,6 +81,20 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
                      int32_t *row_blocks, int32_t *row_offsets,
                      int32_t *col_blocks, int32_t *col_offsets,
                      int32_t *nnz_out, void *workspace, void *stream);
+
+/* ---- dense matrix <-> stack of its stored blocks ---------------------------
+ * Replace SparseLayout.to_sparse / to_dense (sparse/layout.py:40-57).
+ *   dense   [batches, 32 * mask_rows, 32 * mask_cols], contiguous
+ *   sparse  [batches, nnz, 32, 32]
+ *   bsa_to_sparse copies the stored blocks out of `dense` (row_blocks: the row table);
+ *   bsa_to_dense writes every cell of `dense`: the stored blocks, zeros elsewhere
+ *   (`mask` as given to bsa_layout_build, `ordinals` its workspace afterwards).
+ * dtype: BSA_F32 or BSA_F16 (any 4- or 2-byte element type moves the same way).
+ */
+int bsa_to_sparse(int dtype, const void *dense, void *sparse, const int32_t *row_blocks,
+                  int mask_rows, int mask_cols, int nnz, int batches, void *stream);
+int bsa_to_dense(int dtype, const void *sparse, void *dense, const uint8_t *mask, const int32_t *ordinals,
+                 int mask_rows, int mask_cols, int nnz, int batches, void *stream);
 
 /* ---- wavefront schedule -------------------------------------------------
  * Splits every group of a table into chunks of about `cap` pairs, one chunk

@@ -167,3 +167,40 @@ def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices):
         covered[offs[g]: offs[g + 1]] += 1
     assert np.all(covered[: int(offs[-1])] == 1)
     assert last_sliced_wg < first_other_wg                      # sliced rows fill workgroups of their own, first
+
+
+@pytest.mark.parametrize("name,mask", _more_masks())
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.float64])
+def test_to_sparse_to_dense_on_device(name, mask, dtype):
+    """fp16 / fp32 go through the copy kernels, float64 through the torch gather: both must equal the
+    slice definition, and to_dense must write zeros where no block is stored."""
+    mask = np.asarray(mask)
+    if mask.size > 4096:
+        pytest.skip("dense matrix too large for a quick test")
+    L = _layout(mask)
+    r, c = mask.shape
+    g = torch.Generator().manual_seed(r * 131 + c)
+    x = torch.randn(2, 3, 32 * r, 32 * c, generator=g).to(dtype)
+    s = L.to_sparse(x.cuda())
+    assert s.dtype == dtype and tuple(s.shape) == (2, 3, L.num_blocks, 32, 32)
+    assert np.array_equal(s.cpu().numpy(), lo.to_sparse(mask, x.numpy()))
+    d = L.to_dense(s)
+    assert tuple(d.shape) == tuple(x.shape)
+    assert np.array_equal(d.cpu().numpy(), lo.to_dense(mask, lo.to_sparse(mask, x.numpy()), 0.0))
+    # no batch dimension, and a non-contiguous view
+    assert np.array_equal(L.to_sparse(x[0, 1].cuda()).cpu().numpy(), lo.to_sparse(mask, x[0, 1].numpy()))
+    xt = x.cuda().transpose(0, 1)
+    assert np.array_equal(L.to_sparse(xt).cpu().numpy(), lo.to_sparse(mask, xt.cpu().numpy()))
+
+
+def test_to_sparse_to_dense_gradients():
+    mask = np.asarray(dict(mask_zoo())["rand16"])
+    L = _layout(mask)
+    x = torch.randn(2, 512, 512, device="cuda", requires_grad=True)
+    w = torch.randn(2, L.num_blocks, 32, 32, device="cuda")
+    (L.to_sparse(x) * w).sum().backward()
+    assert torch.equal(x.grad, L.to_dense(w))                   # gradient of a gather is the scatter, zeros elsewhere
+    s = torch.randn(2, L.num_blocks, 32, 32, device="cuda", requires_grad=True)
+    u = torch.randn(2, 512, 512, device="cuda")
+    (L.to_dense(s) * u).sum().backward()
+    assert torch.equal(s.grad, L.to_sparse(u))
