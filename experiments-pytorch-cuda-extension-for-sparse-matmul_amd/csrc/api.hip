@@ -77,8 +77,8 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
 static int check_block_copy(const char *who, int dtype, const void *a, const void *b, const void *t0, const void *t1,
                             int mask_rows, int mask_cols, int nnz, int batches)
 {
-    if (dtype != BSA_F32 && dtype != BSA_F16)
-        return fail(BSA_ERR_UNSUPPORTED, "%s: unsupported dtype %d (fp32 = 0, fp16 = 1)", who, dtype);
+    if (dtype != BSA_F32 && dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: unsupported dtype %d (fp32 = 0, fp16 = 1, bf16 = 2)", who, dtype);
     if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
         return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
     if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
@@ -94,7 +94,7 @@ int bsa_to_sparse(int dtype, const void *dense, void *sparse, const int32_t *row
     if (nnz == 0 && dense) return BSA_OK;
     int rc = check_block_copy("bsa_to_sparse", dtype, dense, sparse, row_blocks, row_blocks, mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
-    return check_launch(bsa::launch_to_sparse(dtype == BSA_F16 ? 2 : 4, dense, sparse, row_blocks, nnz, batches,
+    return check_launch(bsa::launch_to_sparse(dtype == BSA_F32 ? 4 : 2, dense, sparse, row_blocks, nnz, batches,
                                               mask_rows, mask_cols, (hipStream_t)stream), "bsa_to_sparse");
 }
 
@@ -105,7 +105,7 @@ int bsa_to_dense(int dtype, const void *sparse, void *dense, const uint8_t *mask
     if (rc) return rc;
     if ((long long)mask_rows * mask_cols > (1LL << 31) - 8)
         return fail(BSA_ERR_INVALID, "bsa_to_dense: %d x %d cells do not fit the launch", mask_rows, mask_cols);
-    return check_launch(bsa::launch_to_dense(dtype == BSA_F16 ? 2 : 4, sparse, dense, mask, ordinals, nnz, batches,
+    return check_launch(bsa::launch_to_dense(dtype == BSA_F32 ? 4 : 2, sparse, dense, mask, ordinals, nnz, batches,
                                              mask_rows, mask_cols, (hipStream_t)stream), "bsa_to_dense");
 }
 
@@ -156,8 +156,8 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
 {
     if (mode != BSA_SDD && mode != BSA_DSD && mode != BSA_DDS)
         return fail(BSA_ERR_INVALID, "bsa_matmul: unknown mode %d", mode);
-    if (dtype != BSA_F32 && dtype != BSA_F16)
-        return fail(BSA_ERR_UNSUPPORTED, "bsa_matmul: unsupported dtype %d (fp32 = 0, fp16 = 1)", dtype);
+    if (dtype != BSA_F32 && dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "bsa_matmul: unsupported dtype %d (fp32 = 0, fp16 = 1, bf16 = 2)", dtype);
     // with nnz == 0 the table and the sparse tensor are empty and may be null
     const bool a_needed = nnz > 0 || mode != BSA_DSD, b_needed = nnz > 0 || mode != BSA_DDS;
     const bool c_needed = nnz > 0 || mode != BSA_SDD;
@@ -216,8 +216,8 @@ static int check_softmax(const char *who, int dtype, const void *p0, const void 
                          const int32_t *blocks, const int32_t *offsets, const int32_t *sched,
                          int sched_wgs, int sched_waves, int mask_rows, int mask_cols, int nnz, int batches)
 {
-    if (dtype != BSA_F32 && dtype != BSA_F16)
-        return fail(BSA_ERR_UNSUPPORTED, "%s: unsupported dtype %d (fp32 = 0, fp16 = 1)", who, dtype);
+    if (dtype != BSA_F32 && dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: unsupported dtype %d (fp32 = 0, fp16 = 1, bf16 = 2)", who, dtype);
     if (!p0 || !p1 || !p2 || !blocks || !offsets) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
     if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
         return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
@@ -262,7 +262,8 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
                           float scale, int causal, void *stream)
 {
     const char *who = "bsa_attention_forward";
-    if (dtype != BSA_F16) return fail(BSA_ERR_UNSUPPORTED, "%s: only fp16 (dtype 1) is built, got %d", who, dtype);
+    if (dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: only fp16 (dtype 1) and bf16 (dtype 2) are built, got %d", who, dtype);
     if (head_dim != 64) return fail(BSA_ERR_UNSUPPORTED, "%s: only head_dim 64 is built, got %d", who, head_dim);
     if (!q || !k || !v || !out || !row_offsets || (!row_blocks && nnz > 0))
         return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
@@ -274,7 +275,7 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
     int rc = check_schedule(sched, sched_wgs, sched_waves, batches, who);
     if (rc) return rc;
     bsa::AttentionArgs p{q, k, v, out, row_blocks, sched, mask_rows, sched_wgs, sched_waves,
-                         mask_rows, mask_cols, batches, scale, causal != 0};
+                         mask_rows, mask_cols, batches, scale, causal != 0, dtype == BSA_BF16};
     return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
 }
 

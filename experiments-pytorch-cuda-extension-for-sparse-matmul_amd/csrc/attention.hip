@@ -41,6 +41,7 @@ __device__ __forceinline__ float at_lane_xor32(float x)
 }
 __device__ __forceinline__ float at_finite_or_zero(float m) { return m == -__builtin_inff() ? 0.f : m; }
 
+template <bool BF>
 __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
     half_t *__restrict__ out, const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
@@ -100,16 +101,16 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
             for (int s = 0; s < 2; ++s)
-                if (!AT_ABLATE(2)) sacc = mfma_f16(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
+                if (!AT_ABLATE(2)) sacc = mfma_16<BF>(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
         if (AT_ABLATE(1)) {
             h8 pq[2];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) pq[i >> 3][i & 7] = (half_t)sacc[i];
+            for (int i = 0; i < 16; ++i) pq[i >> 3][i & 7] = narrow_16<BF>(sacc[i]);
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
-                    if (!AT_ABLATE(4)) oacc[t] = mfma_f16(lds_get_strip<false>(tile_v, 32 * t, s), pq[s], oacc[t]);
+                    if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v, 32 * t, s), pq[s], oacc[t]);
             return;
         }
 
@@ -160,15 +161,15 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         for (int i = 0; i < 16; ++i) {
             const float pv = at_exp2(__builtin_fmaf(sacc[i], mul, -mm));
             psum += pv;
-            pop[i >> 3][i & 7] = (half_t)pv;
+            pop[i >> 3][i & 7] = narrow_16<BF>(pv);
         }
         lsum += psum;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int s = 0; s < 2; ++s)
-                if (!AT_ABLATE(4)) oacc[t] = mfma_f16(lds_get_strip<false>(tile_v, 32 * t, s), pop[s], oacc[t]);
-                else oacc[t][s] += (float)pop[s][0];
+                if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v, 32 * t, s), pop[s], oacc[t]);
+                else oacc[t][s] += widen_16<BF>(pop[s][0]);
     };
 
     // One block in flight: its tiles are requested as soon as the previous block's have been copied
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         for (int g = 0; g < 4; ++g) {
             h4 o;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) o[j] = (half_t)(oacc[t][4 * g + j] * inv);
+            for (int j = 0; j < 4; ++j) o[j] = narrow_16<BF>(oacc[t][4 * g + j] * inv);
             *reinterpret_cast<h4 *>(orow + 32 * t + 8 * g) = o;
         }
     }
@@ -244,10 +245,13 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t st)
 {
     dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
-    attention_fwd_f16_kernel<<<grid, block, (size_t)p.sched_waves * AT_LDS_PER_WAVE, st>>>(
-        (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (half_t *)p.out,
-        (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches,
-        32 * p.mask_rows, 32 * p.mask_cols, p.scale * 1.4426950408889634f, p.causal ? 1 : 0);
+#define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (half_t *)p.out, \
+                    (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
+                    32 * p.mask_rows, 32 * p.mask_cols, p.scale * 1.4426950408889634f, p.causal ? 1 : 0
+    const size_t lds = (size_t)p.sched_waves * AT_LDS_PER_WAVE;
+    if (p.bf16) attention_fwd_f16_kernel<true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+    else attention_fwd_f16_kernel<false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+#undef BSA_AT_ARGS
     return hipGetLastError();
 }
 

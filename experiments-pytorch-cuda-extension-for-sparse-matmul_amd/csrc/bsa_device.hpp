@@ -18,6 +18,7 @@ typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef __fp16 tr4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 
 constexpr int BS = 32;          // block edge
 constexpr int BS2 = BS * BS;    // elements per block
@@ -133,6 +134,27 @@ __device__ __forceinline__ f16v mfma_f16(h8 a, h8 b, f16v c)
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+// 16-bit operands travel as h8 whatever they mean (tiles, LDS maps and requests only see 16-bit
+// elements); BF tells the matrix core and the conversions that the bits are bfloat16.
+template <bool BF>
+__device__ __forceinline__ f16v mfma_16(h8 a, h8 b, f16v c)
+{
+    if (BF) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+template <bool BF>
+__device__ __forceinline__ half_t narrow_16(float x)      // fp32 -> the 16-bit storage type, round to nearest even
+{
+    if (BF) return __builtin_bit_cast(half_t, (__bf16)x);
+    return (half_t)x;
+}
+template <bool BF>
+__device__ __forceinline__ float widen_16(half_t x)
+{
+    if (BF) return (float)__builtin_bit_cast(__bf16, x);
+    return (float)x;
+}
+
 __device__ __forceinline__ f16v mfma_f32(float a, float b, f16v c)
 {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
@@ -157,14 +179,15 @@ __device__ __forceinline__ void stg16_stream(void *p, uint4 v)
 
 __device__ __forceinline__ h8 as_h8(uint4 v) { return __builtin_bit_cast(h8, v); }
 
-// 16 fp32 accumulators -> 16 halves in two 16-byte registers.
+// 16 fp32 accumulators -> 16 halves (or bfloat16) in two 16-byte registers.
+template <bool BF = false>
 __device__ __forceinline__ void pack16(const f16v &acc, uint4 &lo, uint4 &hi)
 {
     h8 a, b;
 #pragma unroll
     for (int v = 0; v < 8; ++v) {
-        a[v] = (half_t)acc[v];
-        b[v] = (half_t)acc[v + 8];
+        a[v] = narrow_16<BF>(acc[v]);
+        b[v] = narrow_16<BF>(acc[v + 8]);
     }
     lo = __builtin_bit_cast(uint4, a);
     hi = __builtin_bit_cast(uint4, b);

@@ -65,6 +65,7 @@ struct AttentionArgs {
     int mask_rows, mask_cols, batches;
     float scale;
     bool causal;
+    bool bf16;      // operands are bfloat16, not fp16
 };
 
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t stream);

@@ -76,7 +76,7 @@ constexpr int SDD_LDS_PER_WAVE = 2048 * (1 + SDD_KB_MAX);   // a / result tile +
 // ---------------------------------------------------------------------------
 // SDD fp16
 // ---------------------------------------------------------------------------
-template <bool A_KC, bool B_KC, int KBT>
+template <bool A_KC, bool B_KC, int KBT, bool BF>
 __global__ __launch_bounds__(512) void sdd_f16_kernel(
     const half_t *__restrict__ a, const half_t *__restrict__ b, half_t *__restrict__ c,
     const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
     // with 16 consecutive columns of its row; the block leaves through LDS as whole 2 KB
     auto store = [&](int idx, const f16v &acc) {
         uint4 lo, hi, raw[2];
-        pack16(acc, lo, hi);
+        pack16<BF>(acc, lo, hi);
         wave_lds_fence();
         lds_put_result(tile_c, lo, hi);
         wave_lds_fence();
@@ -162,8 +162,8 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
                         f16v acc = {0};
 #pragma unroll
                         for (int kb = 0; kb < KB; ++kb) {
-                            acc = mfma_f16(get_b(tile_b + kb * BS2, 0), aop[kb][0], acc);
-                            acc = mfma_f16(get_b(tile_b + kb * BS2, 1), aop[kb][1], acc);
+                            acc = mfma_16<BF>(get_b(tile_b + kb * BS2, 0), aop[kb][0], acc);
+                            acc = mfma_16<BF>(get_b(tile_b + kb * BS2, 1), aop[kb][1], acc);
                         }
                         store(d[u].idx, acc);
                     }
@@ -189,8 +189,8 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
                     load_a(kb + 1, araw);
                     load_b(d.col(), kb + 1, braw);
                 }
-                acc = mfma_f16(get_b(tile_b, 0), get_a(tile_a, 0), acc);
-                acc = mfma_f16(get_b(tile_b, 1), get_a(tile_a, 1), acc);
+                acc = mfma_16<BF>(get_b(tile_b, 0), get_a(tile_a, 0), acc);
+                acc = mfma_16<BF>(get_b(tile_b, 1), get_a(tile_a, 1), acc);
             }
             store(d.idx, acc);
         }
@@ -362,7 +362,7 @@ __device__ __forceinline__ bool split_combine(f16v (&acc)[2], const SchedEntry &
     return true;
 }
 
-template <bool S_KC, bool D_KC, bool DSD, int DEPTH>
+template <bool S_KC, bool D_KC, bool DSD, int DEPTH, bool BF>
 __global__ __launch_bounds__(512) void gw_f16_kernel(
     const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
     const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
@@ -441,7 +441,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
                 if (t < ytiles) {
                     const h8 dop = D_KC ? lds_get_kc(tile_d + t * BS2, s)
                                         : lds_get_strip<DSD>(tile_d, 32 * t, s);
-                    acc[t] = DSD ? mfma_f16(dop, sop, acc[t]) : mfma_f16(sop, dop, acc[t]);
+                    acc[t] = DSD ? mfma_16<BF>(dop, sop, acc[t]) : mfma_16<BF>(sop, dop, acc[t]);
                 }
             }
         }
@@ -481,7 +481,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
         for (int t = 0; t < 2; ++t) {
             if (t < ytiles) {
                 uint4 lo, hi;
-                pack16(acc[t], lo, hi);
+                pack16<BF>(acc[t], lo, hi);
                 half_t *o = ob + gw_out_offset<DSD>(e.group, y0, t, l, DN, XT);
                 stg16(o, lo);
                 stg16(o + 8, hi);
@@ -553,7 +553,7 @@ static inline unsigned grid_x(int n_swg, int batches) { return 8u * (unsigned)n_
 static inline const SchedGroup *sched_groups(const MatmulArgs &p) { return (const SchedGroup *)p.sched; }
 static inline const SchedEntry *sched_slots(const MatmulArgs &p) { return (const SchedEntry *)p.sched + p.groups; }
 
-template <bool A_KC, bool B_KC>
+template <bool A_KC, bool B_KC, bool BF>
 static hipError_t launch_sdd_f16(const MatmulArgs &p, hipStream_t st)
 {
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
@@ -561,11 +561,11 @@ static hipError_t launch_sdd_f16(const MatmulArgs &p, hipStream_t st)
 #define BSA_SDD_ARGS (const half_t *)p.a, (const half_t *)p.b, (half_t *)p.c, (const BlockDesc *)p.blocks, \
                      sched_slots(p), p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K
     switch (p.K / BS) {
-        case 1: sdd_f16_kernel<A_KC, B_KC, 1><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
-        case 2: sdd_f16_kernel<A_KC, B_KC, 2><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
-        case 3: sdd_f16_kernel<A_KC, B_KC, 3><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
-        case 4: sdd_f16_kernel<A_KC, B_KC, 4><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
-        default: sdd_f16_kernel<A_KC, B_KC, 0><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        case 1: sdd_f16_kernel<A_KC, B_KC, 1, BF><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        case 2: sdd_f16_kernel<A_KC, B_KC, 2, BF><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        case 3: sdd_f16_kernel<A_KC, B_KC, 3, BF><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        case 4: sdd_f16_kernel<A_KC, B_KC, 4, BF><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        default: sdd_f16_kernel<A_KC, B_KC, 0, BF><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
     }
 #undef BSA_SDD_ARGS
     return hipGetLastError();
@@ -587,8 +587,12 @@ hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t st)
     // op(b) is K x N: stored [N][K] (contraction contiguous) only with tr_b.
     const bool a_kc = !p.tr_a, b_kc = p.tr_b;
     if (dtype == BSA_F16) {
-        if (a_kc) return b_kc ? launch_sdd_f16<true, true>(p, st) : launch_sdd_f16<true, false>(p, st);
-        return b_kc ? launch_sdd_f16<false, true>(p, st) : launch_sdd_f16<false, false>(p, st);
+        if (a_kc) return b_kc ? launch_sdd_f16<true, true, false>(p, st) : launch_sdd_f16<true, false, false>(p, st);
+        return b_kc ? launch_sdd_f16<false, true, false>(p, st) : launch_sdd_f16<false, false, false>(p, st);
+    }
+    if (dtype == BSA_BF16) {
+        if (a_kc) return b_kc ? launch_sdd_f16<true, true, true>(p, st) : launch_sdd_f16<true, false, true>(p, st);
+        return b_kc ? launch_sdd_f16<false, true, true>(p, st) : launch_sdd_f16<false, false, true>(p, st);
     }
     if (a_kc) return b_kc ? launch_sdd_f32<true, true>(p, st) : launch_sdd_f32<true, false>(p, st);
     return b_kc ? launch_sdd_f32<false, true>(p, st) : launch_sdd_f32<false, false>(p, st);
@@ -607,7 +611,11 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
     ws.counters = (int *)p.workspace;
     ws.tiles = (float *)((char *)p.workspace + gw_counter_bytes(p.split_groups, p.batches, DN));
     if (dtype == BSA_F16)
-        gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH><<<grid, block, lds, st>>>(
+        gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false><<<grid, block, lds, st>>>(
+            (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
+            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+    else if (dtype == BSA_BF16)
+        gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, true><<<grid, block, lds, st>>>(
             (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
             sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
     else

@@ -80,6 +80,54 @@ template <> struct Chunk<half_t> {
         r = __builtin_bit_cast(uint4, h);
     }
 };
+// bfloat16: the same 16-byte chunks as fp16; a value widens by a 16-bit shift and narrows with
+// v_cvt_pk_bf16_f32 (round to nearest even).  No packed min / max for this type.
+struct bf16_t { unsigned short bits; };
+template <> struct Chunk<bf16_t> {
+    static constexpr int NQ = 2;
+    static constexpr int EPC = 8;
+    static constexpr int LPR = 4;
+    static __device__ __forceinline__ void unpack(const uint4 &r, float (&v)[8])
+    {
+        const unsigned w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+        }
+    }
+    static __device__ __forceinline__ uint4 pack(const float (&v)[8])
+    {
+        bf8 h;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[i] = (__bf16)v[i];
+        return __builtin_bit_cast(uint4, h);
+    }
+    static __device__ __forceinline__ void minmax(const uint4 &r, float &lo, float &hi)
+    {
+        float v[8];
+        unpack(r, v);
+        hi = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+        lo = fminf(fminf(fminf(v[0], v[1]), fminf(v[2], v[3])), fminf(fminf(v[4], v[5]), fminf(v[6], v[7])));
+    }
+    static __device__ __forceinline__ uint4 scaled(const uint4 &r, float f)
+    {
+        float v[8];
+        unpack(r, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] *= f;
+        return pack(v);
+    }
+    static __device__ __forceinline__ void mask_right_of(uint4 &r, int col0, int limit, float fill)
+    {
+        float v[8];
+        unpack(r, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (col0 + i > limit) v[i] = fill;
+        r = pack(v);
+    }
+};
 template <> struct Chunk<float> {
     static constexpr int NQ = 4;
     static constexpr int EPC = 4;
@@ -871,6 +919,10 @@ hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t s
         softmax_fwd_kernel<half_t, 4, 48><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (half_t *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
+    else if (dtype == BSA_BF16)
+        softmax_fwd_kernel<bf16_t, 4, 48><<<grid, block, 0, st>>>(
+            (const bf16_t *)p.x, (bf16_t *)p.out, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, scale2, p.causal ? 1 : 0);
     else
         softmax_fwd_kernel<float, 2, 24><<<grid, block, 0, st>>>(
             (const float *)p.x, (float *)p.out, (const BlockDesc *)p.blocks,
@@ -884,6 +936,10 @@ hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t 
     if (dtype == BSA_F16)
         softmax_bwd_kernel<half_t, 2, 24><<<grid, block, 0, st>>>(
             (const half_t *)p.x, (const half_t *)p.dy, (half_t *)p.out, (const BlockDesc *)p.blocks,
+            (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
+    else if (dtype == BSA_BF16)
+        softmax_bwd_kernel<bf16_t, 2, 24><<<grid, block, 0, st>>>(
+            (const bf16_t *)p.x, (const bf16_t *)p.dy, (bf16_t *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     else
         softmax_bwd_kernel<float, 1, 12><<<grid, block, 0, st>>>(

@@ -20,10 +20,10 @@ SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split acro
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
-SOFTMAX_SLICE_MAX = {torch.float16: (48, 24), torch.float32: (24, 12)}
+SOFTMAX_SLICE_MAX = {torch.float16: (48, 24), torch.bfloat16: (48, 24), torch.float32: (24, 12)}
 SOFTMAX_SLICES = (4, 4)              # forward, backward
 
-_DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
+_DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16, torch.bfloat16: _k.BSA_BF16}
 
 
 class Schedule:
@@ -109,7 +109,7 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
     if mode not in _k.MODES:
         raise ValueError(f"mode must be one of 'sdd', 'dsd', 'dds', got {mode!r}")
     if a.dtype != b.dtype or a.dtype not in _DTYPES:
-        raise TypeError(f"operands must both be float32 or both float16, got {a.dtype} and {b.dtype}")
+        raise TypeError(f"operands must both be float32, float16 or bfloat16, got {a.dtype} and {b.dtype}")
     if not (a.is_cuda and b.is_cuda) or a.device != b.device:
         raise ValueError("operands must live on the same GPU")
     _check_layout(row_layout, "row_layout")
@@ -175,7 +175,7 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
 
 def _softmax_common(x, row_layout, col_layout, name):
     if x.dtype not in _DTYPES:
-        raise TypeError(f"{name} must be float32 or float16, got {x.dtype}")
+        raise TypeError(f"{name} must be float32, float16 or bfloat16, got {x.dtype}")
     if not x.is_cuda:
         raise ValueError(f"{name} must live on the GPU")
     _check_layout(row_layout, "row_layout")
@@ -233,8 +233,8 @@ def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=F
     row_layout = (row_blocks, row_table)
     _check_layout(row_layout, "row_layout")
     for t, name in ((q, "q"), (k, "k"), (v, "v")):
-        if t.dtype != torch.float16:
-            raise TypeError(f"{name} must be float16, got {t.dtype}")
+        if t.dtype not in (torch.float16, torch.bfloat16) or t.dtype != q.dtype:
+            raise TypeError(f"q, k, v must all be float16 or all bfloat16, got {name}: {t.dtype}")
         if not t.is_cuda or t.device != q.device:
             raise ValueError("q, k, v must live on the same GPU")
         if t.dim() < 3:

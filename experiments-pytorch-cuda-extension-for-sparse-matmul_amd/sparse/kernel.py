@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 LIBRARY_PATH = os.path.join(_CSRC, "libbsa_hip.so")
 
-BSA_F32, BSA_F16 = 0, 1
+BSA_F32, BSA_F16, BSA_BF16 = 0, 1, 2
 BSA_SDD, BSA_DSD, BSA_DDS = 0, 1, 2
 MODES = {"sdd": BSA_SDD, "dsd": BSA_DSD, "dds": BSA_DDS}
 

@@ -17,7 +17,7 @@ import torch
 from . import kernel as _k
 
 BLOCK = 32
-_COPY_DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16}
+_COPY_DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16, torch.bfloat16: _k.BSA_BF16}
 
 
 class _BlockCopy(torch.autograd.Function):

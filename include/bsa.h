@@ -44,7 +44,7 @@ extern "C" {
 
 #define BSA_BLOCK 32
 
-enum bsa_dtype { BSA_F32 = 0, BSA_F16 = 1 };
+enum bsa_dtype { BSA_F32 = 0, BSA_F16 = 1, BSA_BF16 = 2 };   /* bf16: fp32 accumulation, like fp16 */
 enum bsa_mode { BSA_SDD = 0, BSA_DSD = 1, BSA_DDS = 2 };
 
 enum bsa_status {
@@ -89,7 +89,7 @@ int bsa_layout_build(const uint8_t *mask, int mask_rows, int mask_cols,
  *   bsa_to_sparse copies the stored blocks out of `dense` (row_blocks: the row table);
  *   bsa_to_dense writes every cell of `dense`: the stored blocks, zeros elsewhere
  *   (`mask` as given to bsa_layout_build, `ordinals` its workspace afterwards).
- * dtype: BSA_F32 or BSA_F16 (any 4- or 2-byte element type moves the same way).
+ * dtype: BSA_F32, BSA_F16 or BSA_BF16 (any 4- or 2-byte element type moves the same way).
  */
 int bsa_to_sparse(int dtype, const void *dense, void *sparse, const int32_t *row_blocks,
                   int mask_rows, int mask_cols, int nnz, int batches, void *stream);
@@ -146,7 +146,7 @@ int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
  *   every launch leaves it zero again, so it can be reused by later launches
  *   on the same stream (launches that overlap in time need separate ones).
  *   SDD takes no workspace (null, 0).
- * fp16 accumulates in fp32.  Empty groups give zero rows / columns.
+ * fp16 and bf16 accumulate in fp32.  Empty groups give zero rows / columns.
  */
 size_t bsa_matmul_workspace_bytes(int mode, int sched_tile_slots, int sched_split_groups,
                                   int batches, int M, int N);
@@ -167,7 +167,7 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
  * are those of the ROW layout.  Rows with nothing unmasked yield zeros.
  *   forward : y  = softmax_row(scale * x)
  *   backward: dx = scale * (dy - sum_row(dy * y)) * y
- * Math is fp32 for both dtypes.
+ * Math is fp32 for every dtype.
  */
 int bsa_softmax_forward(int dtype, const void *x, void *y,
                         const int32_t *row_blocks, const int32_t *row_offsets,
@@ -191,7 +191,7 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
  *   out  [batches, 32 * mask_rows, head_dim]; rows without stored (or unmasked) blocks give zeros
  *   tables / schedule: those of the ROW layout; the schedule must be built with
  *   allow_split = 0 and slice_max = -1 (a block row stays inside one workgroup).
- * fp16 only (BSA_ERR_UNSUPPORTED otherwise), head_dim 64.
+ * fp16 and bf16 only (BSA_ERR_UNSUPPORTED otherwise), head_dim 64.
  */
 int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out,
                           const int32_t *row_blocks, const int32_t *row_offsets,
