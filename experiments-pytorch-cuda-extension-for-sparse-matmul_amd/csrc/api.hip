@@ -151,7 +151,7 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
                const int32_t *sched, int sched_wgs, int sched_waves,
                int sched_tile_slots, int sched_split_groups,
                void *workspace, size_t workspace_bytes,
-               int mask_rows, int mask_cols, int nnz, int batches,
+               int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
                int M, int N, int K, int tr_a, int tr_b, void *stream)
 {
     if (mode != BSA_SDD && mode != BSA_DSD && mode != BSA_DDS)
@@ -168,6 +168,9 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
     if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
         return fail(BSA_ERR_INVALID, "bsa_matmul: nnz %d does not fit a %d x %d mask", nnz, mask_rows, mask_cols);
     if (batches < 1) return fail(BSA_ERR_INVALID, "bsa_matmul: batches %d < 1", batches);
+    if (sparse_batches != batches && (sparse_batches != 1 || mode == BSA_SDD))
+        return fail(BSA_ERR_INVALID, "bsa_matmul: sparse_batches must equal batches (%d), or be 1 for dsd / dds; got %d",
+                    batches, sparse_batches);
     if (M < 1 || N < 1 || K < 1 || M % BSA_BLOCK || N % BSA_BLOCK || K % BSA_BLOCK)
         return fail(BSA_ERR_INVALID, "bsa_matmul: M, N, K = %d, %d, %d must be positive multiples of %d", M, N, K, BSA_BLOCK);
     int rc = check_schedule(sched, sched_wgs, sched_waves, batches, "bsa_matmul");
@@ -205,7 +208,7 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
         return fail(BSA_ERR_INVALID, "bsa_matmul: workspace of %zu bytes needed, %zu given", ws_need, workspace_bytes);
 
     bsa::MatmulArgs p{a, b, c, blocks, sched, groups, sched_wgs, sched_waves, sched_tile_slots, sched_split_groups,
-                      workspace, nnz, batches, M, N, K, tr_a != 0, tr_b != 0};
+                      workspace, nnz, batches, M, N, K, tr_a != 0, tr_b != 0, sparse_batches != batches};
     if (nnz == 0 && mode == BSA_SDD) return BSA_OK;   // nothing to write
     hipError_t err = mode == BSA_SDD ? bsa::launch_sdd(dtype, p, (hipStream_t)stream)
                                      : bsa::launch_group_walk(dtype, mode == BSA_DSD, p, (hipStream_t)stream);

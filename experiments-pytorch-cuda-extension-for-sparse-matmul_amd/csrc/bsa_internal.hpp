@@ -31,6 +31,7 @@ struct MatmulArgs {
     int nnz, batches;
     int M, N, K;
     bool tr_a, tr_b;
+    bool sparse_shared;   // DSD / DDS: the sparse operand has no batch dimension
 };
 
 hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t stream);

@@ -367,7 +367,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
     const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
     const SchedEntry *__restrict__ sched, SplitWorkspace ws,
-    int n_swg, int batches, int nnz, int DN, int KT, int XT)
+    int n_swg, int batches, int nnz, int DN, int KT, int XT, int sp_shared)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     BSA_TRACE_BEGIN
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
 
     half_t *tile_s = reinterpret_cast<half_t *>(lds_raw + (size_t)w * GW_LDS_PER_WAVE);
     half_t *tile_d = tile_s + BS2;
-    const half_t *spb = sp + (size_t)batch * nnz * BS2;
+    const half_t *spb = sp + (sp_shared ? 0 : (size_t)batch * nnz * BS2);   // one sparse operand for the whole batch?
     const half_t *dnb = dn + (size_t)batch * DN * KT;
 
     // one pair's operands: 2 KB of the sparse block + up to 4 KB of the dense strip,
@@ -496,7 +496,7 @@ __global__ __launch_bounds__(512) void gw_f32_kernel(
     const float *__restrict__ sp, const float *__restrict__ dn, float *__restrict__ out,
     const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
     const SchedEntry *__restrict__ sched, SplitWorkspace ws,
-    int n_swg, int batches, int nnz, int DN, int KT, int XT)
+    int n_swg, int batches, int nnz, int DN, int KT, int XT, int sp_shared)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int batch, swg;
@@ -506,7 +506,7 @@ __global__ __launch_bounds__(512) void gw_f32_kernel(
     const SchedEntry e = sched[swg * W + w];
     const int y0 = 64 * (int)blockIdx.y;
     const int ytiles = (DN - y0) >= 64 ? 2 : 1;
-    const float *spb = sp + (size_t)batch * nnz * BS2;
+    const float *spb = sp + (sp_shared ? 0 : (size_t)batch * nnz * BS2);
     const float *dnb = dn + (size_t)batch * DN * KT;
 
     f16v acc[2] = {{0}, {0}};
@@ -613,15 +613,15 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
     if (dtype == BSA_F16)
         gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false><<<grid, block, lds, st>>>(
             (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
-            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
     else if (dtype == BSA_BF16)
         gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, true><<<grid, block, lds, st>>>(
             (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
-            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
     else
         gw_f32_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(
             (const float *)sp, (const float *)dn, (float *)p.c, (const BlockDesc *)p.blocks,
-            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT);
+            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
     return hipGetLastError();
 }
 

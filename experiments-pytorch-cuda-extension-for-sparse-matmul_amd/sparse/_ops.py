@@ -126,9 +126,13 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
     sparse_width = (layout[1].numel() - 1) * BLOCK                      # :14
 
     a_dense, b_dense = mode[1] == "d", mode[2] == "d"
-    if a.dim() < (3 if a_dense else 4) or b.dim() < (3 if b_dense else 4):
+    # a sparse INPUT without batch dimensions is shared by every batch entry of the dense operand
+    shared = (not a_dense and a.dim() == 3) or (not b_dense and b.dim() == 3)
+    if (a_dense and a.dim() < 3) or (b_dense and b.dim() < 3) or (not a_dense and a.dim() < 3) \
+            or (not b_dense and b.dim() < 3):
         raise ValueError("operands need at least one batch dimension "
-                         "(dense [..., rows, cols], sparse [..., nnz, 32, 32])")
+                         "(dense [..., rows, cols], sparse [..., nnz, 32, 32]; a sparse input may "
+                         "also be [nnz, 32, 32], shared by the whole batch)")
     for t, dense, name in ((a, a_dense, "a"), (b, b_dense, "b")):
         if not dense and tuple(t.shape[-3:]) != (num_blocks, BLOCK, BLOCK):
             raise ValueError(f"sparse operand {name} must be [..., {num_blocks}, 32, 32], got {tuple(t.shape)}")
@@ -142,8 +146,11 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
 
     batch_a = tuple(a.shape[:-2] if a_dense else a.shape[:-3])
     batch_b = tuple(b.shape[:-2] if b_dense else b.shape[:-3])
+    if shared:
+        batch_a = batch_b = batch_a if a_dense else batch_b
     if batch_a != batch_b:
-        raise ValueError(f"batch dimensions differ: {batch_a} vs {batch_b} (no broadcasting)")
+        raise ValueError(f"batch dimensions differ: {batch_a} vs {batch_b} (only a sparse input without "
+                         f"batch dimensions is broadcast)")
     batches = 1
     for s in batch_a:
         batches *= s
@@ -168,7 +175,7 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
             layout[0].data_ptr(), layout[1].data_ptr(), layout[1].numel() - 1,
             sched.table.data_ptr(), sched.workgroups, sched.waves, sched.tile_slots, sched.split_groups,
             ws.data_ptr() if ws is not None else None, ws_bytes,
-            mask_rows, mask_cols, num_blocks, batches, size_m, size_n, size_k,
+            mask_rows, mask_cols, num_blocks, batches, 1 if shared else batches, size_m, size_n, size_k,
             int(trans_a), int(trans_b), stream))
     return c
 

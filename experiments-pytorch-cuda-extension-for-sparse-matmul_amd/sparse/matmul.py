@@ -49,6 +49,11 @@ class SparseMatMul(torch.autograd.Function):
             db = sparse_ops.sparse_matmul(lhs, rhs, db_mode, layout.row_layout, layout.col_layout,
                                           not trans_a or trans_b, trans_a and trans_b)
 
+        # a sparse input given without batch dimensions was shared by the batch: its gradient is the sum
+        if da is not None and da.dim() > a.dim():
+            da = da.sum(dim=tuple(range(da.dim() - a.dim())))
+        if db is not None and db.dim() > b.dim():
+            db = db.sum(dim=tuple(range(db.dim() - b.dim())))
         return da, db, None, None, None, None
 
 

@@ -146,6 +146,8 @@ int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
  *   every launch leaves it zero again, so it can be reused by later launches
  *   on the same stream (launches that overlap in time need separate ones).
  *   SDD takes no workspace (null, 0).
+ *   sparse_batches is `batches`, or 1 (DSD / DDS only) when ONE sparse operand [nnz, 32, 32] serves
+ *   every batch entry (a block-sparse weight); the reference has no such case.
  * fp16 and bf16 accumulate in fp32.  Empty groups give zero rows / columns.
  */
 size_t bsa_matmul_workspace_bytes(int mode, int sched_tile_slots, int sched_split_groups,
@@ -155,7 +157,7 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
                const int32_t *sched, int sched_wgs, int sched_waves,
                int sched_tile_slots, int sched_split_groups,
                void *workspace, size_t workspace_bytes,
-               int mask_rows, int mask_cols, int nnz, int batches,
+               int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
                int M, int N, int K, int tr_a, int tr_b, void *stream);
 
 /* ---- block-sparse softmax ----------------------------------------------

@@ -49,9 +49,10 @@ P = 0x1000  # any non-null address: validation fails before anything is derefere
 
 def _matmul(k, mode=0, dtype=1, a=P, b=P, c=P, blocks=P, offs=P, groups=4, sched=P, wgs=1, waves=4,
             tiles=0, splits=0, ws=None, ws_bytes=0,
-            R=4, C=4, nnz=5, batches=1, M=128, N=128, K=64, ta=0, tb=1):
+            R=4, C=4, nnz=5, batches=1, sparse_batches=None, M=128, N=128, K=64, ta=0, tb=1):
     return k.lib.bsa_matmul(mode, dtype, a, b, c, blocks, offs, groups, sched, wgs, waves, tiles, splits,
-                            ws, ws_bytes, R, C, nnz, batches, M, N, K, ta, tb, None)
+                            ws, ws_bytes, R, C, nnz, batches, batches if sparse_batches is None else sparse_batches,
+                            M, N, K, ta, tb, None)
 
 
 @pytest.mark.parametrize("kw,needle", [
@@ -64,6 +65,8 @@ def _matmul(k, mode=0, dtype=1, a=P, b=P, c=P, blocks=P, offs=P, groups=4, sched
     (dict(groups=3), "groups"),
     (dict(nnz=17), "does not fit"),
     (dict(batches=0), "batches"),
+    (dict(batches=3, sparse_batches=2), "sparse_batches"),
+    (dict(batches=3, sparse_batches=1), "sparse_batches"),          # sdd has no sparse input to share
     (dict(waves=9), "waves per workgroup"),
     (dict(wgs=0), "workgroups"),
     (dict(mode=1, ta=0, tb=0, M=128, K=96, N=64), "op(sparse a)"),

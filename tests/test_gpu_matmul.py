@@ -212,3 +212,36 @@ def test_python_boundary_rejects_misuse():
     with pytest.raises(sparse.kernel.BsaError):
         k48 = torch.randn(1, 96, 48, device="cuda")                                            # K % 32
         sparse_ops.sparse_matmul(k48, k48, "sdd", L.row_layout, L.col_layout, False, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("mode,ta,tb", [(m, x, y) for m in ("dsd", "dds") for x in (False, True) for y in (False, True)])
+def test_sparse_operand_shared_by_the_batch(mode, ta, tb, dtype):
+    """A sparse input without batch dimensions (a block-sparse weight) serves every batch entry; its
+    gradient is the sum over the batch."""
+    import sparse
+    mask = np.asarray(ZOO["long_col_70x3"] if mode == "dds" else ZOO["rand16"])
+    g = torch.Generator().manual_seed(21)
+    sa, sb = operand_shapes(mode, mask, 64, ta, tb, (3,))
+    if mode == "dsd":
+        sa = sa[1:]
+    else:
+        sb = sb[1:]
+    a = torch.randn(sa, generator=g).to(dtype)
+    b = torch.randn(sb, generator=g).to(dtype)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    ad, bd = a.cuda().requires_grad_(True), b.cuda().requires_grad_(True)
+    c = sparse.matmul(ad, bd, mode, L, ta, tb)
+    full_a = a.expand((3,) + tuple(a.shape)) if mode == "dsd" else a
+    full_b = b.expand((3,) + tuple(b.shape)) if mode == "dds" else b
+    ref = mo.matmul(to_np(full_a), to_np(full_b), mode, mask, ta, tb)
+    assert tuple(c.shape) == ref.shape and rel_err(to_np(c), ref) <= tol_of(dtype)
+    dc = torch.randn(c.shape, generator=g).to(dtype)
+    c.backward(dc.cuda())
+    ga, gb = mo.backward(to_np(full_a), to_np(full_b), to_np(dc), mode, mask, ta, tb)
+    if mode == "dsd":
+        ga = ga.sum(axis=0)
+    else:
+        gb = gb.sum(axis=0)
+    assert ad.grad.shape == ad.shape and bd.grad.shape == bd.shape
+    assert rel_err(to_np(ad.grad), ga) <= 2 * tol_of(dtype) and rel_err(to_np(bd.grad), gb) <= 2 * tol_of(dtype)
