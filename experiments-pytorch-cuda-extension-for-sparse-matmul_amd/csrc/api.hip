@@ -267,7 +267,8 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
     const char *who = "bsa_attention_forward";
     if (dtype != BSA_F16 && dtype != BSA_BF16)
         return fail(BSA_ERR_UNSUPPORTED, "%s: only fp16 (dtype 1) and bf16 (dtype 2) are built, got %d", who, dtype);
-    if (head_dim != 64) return fail(BSA_ERR_UNSUPPORTED, "%s: only head_dim 64 is built, got %d", who, head_dim);
+    if (head_dim != 64 && head_dim != 128)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: head_dim 64 and 128 are built, got %d", who, head_dim);
     if (!q || !k || !v || !out || !row_offsets || (!row_blocks && nnz > 0))
         return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
     if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
@@ -278,7 +279,7 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
     int rc = check_schedule(sched, sched_wgs, sched_waves, batches, who);
     if (rc) return rc;
     bsa::AttentionArgs p{q, k, v, out, row_blocks, sched, mask_rows, sched_wgs, sched_waves,
-                         mask_rows, mask_cols, batches, scale, causal != 0, dtype == BSA_BF16};
+                         mask_rows, mask_cols, batches, scale, causal != 0, dtype == BSA_BF16, head_dim};
     return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
 }
 

@@ -30,8 +30,9 @@ namespace bsa {
 #define AT_ABLATE(bit) 0
 #endif
 
-constexpr int AT_HEAD = 64;                    // head dim
-constexpr int AT_LDS_PER_WAVE = 4096 + 4096 + 512;   // K tile pair + V strip (reused: O^T partial 8 KB) + row stats
+// per wave: K tiles (HD / 32 of 2 KB) + V strips (HD / 64 of 4 KB), reused for the O^T partial of the
+// team merge (HD x 32 floats: the same size), + row stats
+constexpr int at_lds_per_wave(int hd) { return 128 * hd + 512; }
 constexpr float AT_LAZY = 8.f;                // log2 of the growth of a row maximum that forces a rescale
 
 __device__ __forceinline__ float at_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -41,7 +42,7 @@ __device__ __forceinline__ float at_lane_xor32(float x)
 }
 __device__ __forceinline__ float at_finite_or_zero(float m) { return m == -__builtin_inff() ? 0.f : m; }
 
-template <bool BF>
+template <int HD, bool BF>
 __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
     half_t *__restrict__ out, const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
@@ -58,9 +59,11 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     const int qq = l & 31, h = l >> 5;          // query column of this lane, lane half
     const float NEG_INF = -__builtin_inff();
 
+    constexpr int AT_HEAD = HD, AT_LDS_PER_WAVE = at_lds_per_wave(HD);
+    constexpr int KT = HD / 32, VS = HD / 64;   // 32-wide K tiles, 64-wide V strips
     unsigned char *my_lds = lds_raw + (size_t)w * AT_LDS_PER_WAVE;
-    half_t *tile_k = reinterpret_cast<half_t *>(my_lds);            // two [key][32 d] tiles
-    half_t *tile_v = reinterpret_cast<half_t *>(my_lds + 4096);     // [key][64 n] strip, rows exchanged
+    half_t *tile_k = reinterpret_cast<half_t *>(my_lds);                 // KT [key][32 d] tiles
+    half_t *tile_v = reinterpret_cast<half_t *>(my_lds + 2048 * KT);     // VS [key][64 n] strips, rows exchanged
     const half_t *kb = k + (size_t)batch * rows_k * AT_HEAD;
     const half_t *vb = v + (size_t)batch * rows_k * AT_HEAD;
 
@@ -72,33 +75,41 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         for (int s = 0; s < AT_HEAD / 16; ++s) qop[s] = as_h8(ldg16(qrow + 16 * s));
     }
 
-    struct Frag { uint4 k0[2], k1[2], vv[4]; };   // K_c as two 32 x 32 tiles (d halves), V_c as a 4 KB strip
+    struct Frag { uint4 kk[KT][2], vv[VS][4]; };   // K_c as 32 x 32 tiles (d slices), V_c as 4 KB strips (n slices)
     DescWindow win;
     auto load = [&](int p, Frag &f) {
         const int c = win.get(p).col();
-        ldg_tile32(kb + (size_t)(BS * c) * AT_HEAD, AT_HEAD, f.k0);
-        ldg_tile32(kb + (size_t)(BS * c) * AT_HEAD + 32, AT_HEAD, f.k1);
+#pragma unroll
+        for (int dt = 0; dt < KT; ++dt) ldg_tile32(kb + (size_t)(BS * c) * AT_HEAD + 32 * dt, AT_HEAD, f.kk[dt]);
         const half_t *vs = vb + (size_t)(BS * c) * AT_HEAD;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) f.vv[t] = ldg16(vs + 8 * (l + 64 * t));
+        for (int u = 0; u < VS; ++u)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int piece = l + 64 * t;               // key row piece / 8, 16-byte piece % 8 of the 128-byte strip row
+                f.vv[u][t] = ldg16(vs + (size_t)(piece >> 3) * AT_HEAD + 64 * u + 8 * (piece & 7));
+            }
     };
 
     float m = NEG_INF, lsum = 0.f;               // running max of the query (both lane halves agree), this half's sum
-    f16v oacc[2] = {{0}, {0}};                   // O^T: lane = query column, values = head dims 32 t + 8 (v / 4) + 4 h + v % 4
+    f16v oacc[KT];                               // O^T: lane = query column, values = head dims 32 t + 8 (v / 4) + 4 h + v % 4
+#pragma unroll
+    for (int t = 0; t < KT; ++t) oacc[t] = f16v{0};
 
     // registers -> staging tiles; the registers are free for the next block's loads afterwards
     auto stage = [&](const Frag &f) {
         if (AT_ABLATE(8)) return;
         wave_lds_fence();
-        lds_put_kc<false>(tile_k, f.k0);
-        lds_put_kc<false>(tile_k + BS2, f.k1);
-        lds_put_strip_swapped(tile_v, f.vv);
+#pragma unroll
+        for (int dt = 0; dt < KT; ++dt) lds_put_kc<false>(tile_k + dt * BS2, f.kk[dt]);
+#pragma unroll
+        for (int u = 0; u < VS; ++u) lds_put_strip_swapped(tile_v + u * 2048, f.vv[u]);
         wave_lds_fence();
     };
     auto step = [&](int c) {
         f16v sacc = {0};
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
+        for (int dt = 0; dt < KT; ++dt)
 #pragma unroll
             for (int s = 0; s < 2; ++s)
                 if (!AT_ABLATE(2)) sacc = mfma_16<BF>(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
@@ -107,10 +118,10 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) pq[i >> 3][i & 7] = narrow_16<BF>(sacc[i]);
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < KT; ++t)
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
-                    if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v, 32 * t, s), pq[s], oacc[t]);
+                    if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v + (t / 2) * 2048, 32 * (t % 2), s), pq[s], oacc[t]);
             return;
         }
 
@@ -150,7 +161,7 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
             m = m_new;
             lsum *= keep;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < KT; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) oacc[t][i] *= keep;
         }
@@ -165,10 +176,10 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         }
         lsum += psum;
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < KT; ++t)
 #pragma unroll
             for (int s = 0; s < 2; ++s)
-                if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v, 32 * t, s), pop[s], oacc[t]);
+                if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v + (t / 2) * 2048, 32 * (t % 2), s), pop[s], oacc[t]);
                 else oacc[t][s] += widen_16<BF>(pop[s][0]);
     };
 
@@ -193,12 +204,13 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     // team merge: every wave but the leader parks (max, sum, O^T); the leader rescales and adds
     const int slot0 = e.first_wave(), nw = e.team_waves();
     const bool leader = active && w == slot0;
-    float *park = reinterpret_cast<float *>(my_lds);                  // 2048 floats of O^T
-    float2 *stat = reinterpret_cast<float2 *>(my_lds + 8192);         // 32 (max, sum)
+    constexpr int STAT_OFF = 128 * HD;                                // behind the HD x 32 floats of O^T
+    float *park = reinterpret_cast<float *>(my_lds);
+    float2 *stat = reinterpret_cast<float2 *>(my_lds + STAT_OFF);     // 32 (max, sum)
     if (active && !leader) {
         wave_lds_fence();
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < KT; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) park[(t * 16 + i) * WAVE + l] = oacc[t][i];
         if (h == 0) stat[qq] = make_float2(m, lsum);
@@ -208,22 +220,22 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     if (nw > 1) {
         float M = m;
         for (int o = 1; o < nw; ++o)
-            M = fmaxf(M, reinterpret_cast<const float2 *>(lds_raw + (size_t)(w + o) * AT_LDS_PER_WAVE + 8192)[qq].x);
+            M = fmaxf(M, reinterpret_cast<const float2 *>(lds_raw + (size_t)(w + o) * AT_LDS_PER_WAVE + STAT_OFF)[qq].x);
         const float MM = at_finite_or_zero(M);
         const float mine = at_exp2(m - MM);
         lsum *= mine;
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < KT; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) oacc[t][i] *= mine;
         for (int o = 1; o < nw; ++o) {
             const unsigned char *other = lds_raw + (size_t)(w + o) * AT_LDS_PER_WAVE;
-            const float2 st = reinterpret_cast<const float2 *>(other + 8192)[qq];
+            const float2 st = reinterpret_cast<const float2 *>(other + STAT_OFF)[qq];
             const float f = at_exp2(st.x - MM);
             lsum += st.y * f;
             const float *op = reinterpret_cast<const float *>(other);
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < KT; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) oacc[t][i] += op[(t * 16 + i) * WAVE + l] * f;
         }
@@ -231,7 +243,7 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
     half_t *orow = out + ((size_t)batch * rows_q + BS * r + qq) * AT_HEAD + 4 * h;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < KT; ++t) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             h4 o;
@@ -248,9 +260,21 @@ hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t st)
 #define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (half_t *)p.out, \
                     (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
                     32 * p.mask_rows, 32 * p.mask_cols, p.scale * 1.4426950408889634f, p.causal ? 1 : 0
-    const size_t lds = (size_t)p.sched_waves * AT_LDS_PER_WAVE;
-    if (p.bf16) attention_fwd_f16_kernel<true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
-    else attention_fwd_f16_kernel<false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+    const size_t lds = (size_t)p.sched_waves * at_lds_per_wave(p.head_dim);
+    if (p.head_dim == 64) {
+        if (p.bf16) attention_fwd_f16_kernel<64, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+        else attention_fwd_f16_kernel<64, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+    } else {
+        // more than 3 waves x 16.5 KB of staging exceed the 64 KB a launch gets without asking
+        if (lds > 65536) {
+            const void *fn = p.bf16 ? (const void *)attention_fwd_f16_kernel<128, true>
+                                    : (const void *)attention_fwd_f16_kernel<128, false>;
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        if (p.bf16) attention_fwd_f16_kernel<128, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+        else attention_fwd_f16_kernel<128, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+    }
 #undef BSA_AT_ARGS
     return hipGetLastError();
 }

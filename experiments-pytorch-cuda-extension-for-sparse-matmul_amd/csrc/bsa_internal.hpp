@@ -67,6 +67,7 @@ struct AttentionArgs {
     float scale;
     bool causal;
     bool bf16;      // operands are bfloat16, not fp16
+    int head_dim;   // 64 or 128
 };
 
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t stream);

@@ -236,7 +236,7 @@ def sparse_softmax_backward(y, dy, row_blocks, row_table, scale=1.0, col_layout=
 def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=False, col_layout=None):
     """``softmax(scale * q k^T on the stored blocks) v`` in one launch: the chain of
     ``sparse_matmul('sdd', trans_b)``, the softmax and ``sparse_matmul('dsd')`` (sparse/matmul.py:57,
-    sparse_softmax.cu:208-231) without the scores in memory.  fp16, head dim 64."""
+    sparse_softmax.cu:208-231) without the scores in memory.  fp16 / bf16, head dim 64 or 128."""
     row_layout = (row_blocks, row_table)
     _check_layout(row_layout, "row_layout")
     for t, name in ((q, "q"), (k, "k"), (v, "v")):

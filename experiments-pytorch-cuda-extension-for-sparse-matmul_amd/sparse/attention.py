@@ -42,6 +42,6 @@ class SparseAttention(torch.autograd.Function):
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, layout: SparseLayout, scale: float = 1.0,
               causal: bool = False) -> torch.Tensor:
-    """``softmax(scale * q @ k^T, over the stored blocks of each row) @ v`` for fp16
-    ``q [..., 32 R, 64]``, ``k``, ``v [..., 32 C, 64]`` and an ``R x C`` block layout."""
+    """``softmax(scale * q @ k^T, over the stored blocks of each row) @ v`` for fp16 / bf16
+    ``q [..., 32 R, D]``, ``k``, ``v [..., 32 C, D]``, ``D`` 64 or 128, and an ``R x C`` block layout."""
     return SparseAttention.apply(q, k, v, layout, scale, causal)

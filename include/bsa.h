@@ -193,7 +193,7 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
  *   out  [batches, 32 * mask_rows, head_dim]; rows without stored (or unmasked) blocks give zeros
  *   tables / schedule: those of the ROW layout; the schedule must be built with
  *   allow_split = 0 and slice_max = -1 (a block row stays inside one workgroup).
- * fp16 and bf16 only (BSA_ERR_UNSUPPORTED otherwise), head_dim 64.
+ * fp16 and bf16 only, head_dim 64 or 128 (BSA_ERR_UNSUPPORTED otherwise).
  */
 int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out,
                           const int32_t *row_blocks, const int32_t *row_offsets,

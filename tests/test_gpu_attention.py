@@ -11,10 +11,10 @@ ZOO = dict(mask_zoo())
 TOL = 2e-3          # fp16 operands, fp32 accumulation, probabilities rounded to fp16 (as in the chain)
 
 
-def _qkv(mask, batch=(2,), seed=0, std=1.0):
+def _qkv(mask, batch=(2,), seed=0, std=1.0, head=64):
     g = torch.Generator().manual_seed(seed)
     r, c = np.asarray(mask).shape
-    mk = lambda n: (std * torch.randn(*batch, 32 * n, 64, generator=g)).half()
+    mk = lambda n: (std * torch.randn(*batch, 32 * n, head, generator=g)).half()
     return mk(r), mk(c), mk(c)
 
 
@@ -32,6 +32,14 @@ def _run(mask, scale, causal, **kw):
                                   "wide_2x9", "rand16", "long_row_5x40", "long_col_70x3"])
 def test_forward(name, scale, causal):
     out, ref = _run(np.asarray(ZOO[name]), scale, causal)
+    assert np.all(np.isfinite(out))
+    assert rel_err(out, ref) <= TOL
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("name", ["known3x3", "empty_row_col_6x5", "rand16", "long_row_5x40", "long_col_70x3"])
+def test_forward_head_dim_128(name, causal):
+    out, ref = _run(np.asarray(ZOO[name]), 0.09, causal, head=128, seed=3)
     assert np.all(np.isfinite(out))
     assert rel_err(out, ref) <= TOL
 
@@ -108,4 +116,4 @@ def test_argument_checks():
     with pytest.raises(ValueError):
         sparse.attention(q[:, :64], k, v, L)
     with pytest.raises(Exception):
-        sparse.attention(q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous(), L)
+        sparse.attention(q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous(), L)   # head dim 32
