@@ -175,6 +175,38 @@ def main():
         attention[name + "_nnz_TFLOPs"] = round(2 * flops_one / (ms * 1e-3) / 1e12, 2)
     attention["speedup"] = round(attention["chain_us"] / attention["fused_us"], 2)
 
+    # the backward pass of the same attention: one launch for P and dS + three products, against the
+    # seven launches of the unfused chain (gradients of q, k, v from dout)
+    from sparse.kernel import sparse_ops
+    rows, cols = layout.row_layout, layout.col_layout
+    for w in sets:
+        w["dout"] = torch.randn_like(w["q"])
+        w["out"], w["lse"] = sparse_ops.sparse_attention_forward(w["q"], w["k"], w["v"], rows[0], rows[1], 0.125, True,
+                                                                 cols, return_lse=True)
+
+    def products(p, ds, w):
+        return (sparse.matmul(ds, w["k"], "dsd", layout), sparse.matmul(ds, w["q"], "dsd", layout, True, False),
+                sparse.matmul(p, w["dout"], "dsd", layout, True, False))
+
+    def backward_fused(w):
+        p, ds = sparse_ops.sparse_attention_backward_scores(w["q"], w["k"], w["v"], w["dout"], w["out"], w["lse"],
+                                                            rows[0], rows[1], 0.125, True, cols)
+        return products(p, ds, w)
+
+    def backward_chain(w):
+        p = sparse.softmax(sparse.matmul(w["q"], w["k"], "sdd", layout, False, True), layout, 0.125, True)
+        dp = sparse.matmul(w["dout"], w["v"], "sdd", layout, False, True)
+        ds = sparse_ops.sparse_softmax_backward(p, dp, rows[0], rows[1], 0.125, cols)
+        return products(p, ds, w)
+
+    with torch.no_grad():
+        for a, b in zip(backward_fused(sets[0]), backward_chain(sets[0])):
+            err = ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+            assert err <= 4e-3, f"attention backward differs from the chain: {err}"
+    for name, fn in (("backward_us", backward_fused), ("backward_chain_us", backward_chain)):
+        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+        attention[name] = round(ms * 1e3, 3)
+
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/): same
     # workload, same kernels; absent file -> null
     traffic = {}
@@ -203,7 +235,7 @@ def main():
                                  "unit": "GB/s", "frac": per_op["softmax"]["hbm_frac"],
                                  "traffic": traffic.get("softmax")}},
         "kernels": per_op,
-        "attention_forward": attention,
+        "attention": attention,
     }
 
     if not args.no_cpu:

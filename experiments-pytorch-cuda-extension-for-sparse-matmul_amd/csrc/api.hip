@@ -258,29 +258,58 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
     return check_launch(bsa::launch_softmax_backward(dtype, p, (hipStream_t)stream), "bsa_softmax_backward");
 }
 
-int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out,
+static int check_attention(const char *who, int dtype, int head_dim, const int32_t *row_blocks,
+                           const int32_t *row_offsets, const int32_t *sched, int sched_wgs, int sched_waves,
+                           int mask_rows, int mask_cols, int nnz, int batches)
+{
+    if (dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: only fp16 (dtype 1) and bf16 (dtype 2) are built, got %d", who, dtype);
+    if (head_dim != 64 && head_dim != 128)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: head_dim 64 and 128 are built, got %d", who, head_dim);
+    if (!row_offsets || (!row_blocks && nnz > 0)) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
+    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
+        return fail(BSA_ERR_INVALID, "%s: nnz %d does not fit a %d x %d mask", who, nnz, mask_rows, mask_cols);
+    if (batches < 1) return fail(BSA_ERR_INVALID, "%s: batches %d < 1", who, batches);
+    return check_schedule(sched, sched_wgs, sched_waves, batches, who);
+}
+
+int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out, float *lse,
                           const int32_t *row_blocks, const int32_t *row_offsets,
                           const int32_t *sched, int sched_wgs, int sched_waves,
                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                           float scale, int causal, void *stream)
 {
     const char *who = "bsa_attention_forward";
-    if (dtype != BSA_F16 && dtype != BSA_BF16)
-        return fail(BSA_ERR_UNSUPPORTED, "%s: only fp16 (dtype 1) and bf16 (dtype 2) are built, got %d", who, dtype);
-    if (head_dim != 64 && head_dim != 128)
-        return fail(BSA_ERR_UNSUPPORTED, "%s: head_dim 64 and 128 are built, got %d", who, head_dim);
-    if (!q || !k || !v || !out || !row_offsets || (!row_blocks && nnz > 0))
-        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
-    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
-        return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
-    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
-        return fail(BSA_ERR_INVALID, "%s: nnz %d does not fit a %d x %d mask", who, nnz, mask_rows, mask_cols);
-    if (batches < 1) return fail(BSA_ERR_INVALID, "%s: batches %d < 1", who, batches);
-    int rc = check_schedule(sched, sched_wgs, sched_waves, batches, who);
+    int rc = check_attention(who, dtype, head_dim, row_blocks, row_offsets, sched, sched_wgs, sched_waves,
+                             mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
-    bsa::AttentionArgs p{q, k, v, out, row_blocks, sched, mask_rows, sched_wgs, sched_waves,
-                         mask_rows, mask_cols, batches, scale, causal != 0, dtype == BSA_BF16, head_dim};
+    if (!q || !k || !v || !out) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    bsa::AttentionArgs p{q, k, v, out, lse, nullptr, nullptr, nullptr, nnz, row_blocks, sched, mask_rows,
+                         sched_wgs, sched_waves, mask_rows, mask_cols, batches, scale, causal != 0,
+                         dtype == BSA_BF16, head_dim};
     return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
+}
+
+int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const void *v, const void *dout,
+                                  const void *out, const float *lse, void *p_out, void *ds_out,
+                                  const int32_t *row_blocks, const int32_t *row_offsets,
+                                  const int32_t *sched, int sched_wgs, int sched_waves,
+                                  int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
+                                  float scale, int causal, void *stream)
+{
+    const char *who = "bsa_attention_backward_scores";
+    int rc = check_attention(who, dtype, head_dim, row_blocks, row_offsets, sched, sched_wgs, sched_waves,
+                             mask_rows, mask_cols, nnz, batches);
+    if (rc) return rc;
+    if (nnz == 0) return BSA_OK;      // no blocks to write
+    if (!q || !k || !v || !dout || !out || !lse || !p_out || !ds_out)
+        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    bsa::AttentionArgs p{q, k, v, const_cast<void *>(out), const_cast<float *>(lse), dout, p_out, ds_out, nnz,
+                         row_blocks, sched, mask_rows, sched_wgs, sched_waves, mask_rows, mask_cols, batches,
+                         scale, causal != 0, dtype == BSA_BF16, head_dim};
+    return check_launch(bsa::launch_attention_backward_scores(p, (hipStream_t)stream), who);
 }
 
 }  // extern "C"

@@ -45,7 +45,8 @@ __device__ __forceinline__ float at_finite_or_zero(float m) { return m == -__bui
 template <int HD, bool BF>
 __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
-    half_t *__restrict__ out, const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    half_t *__restrict__ out, float *__restrict__ lse, const BlockDesc *__restrict__ blocks,
+    const SchedEntry *__restrict__ sched,
     int n_swg, int batches, int rows_q, int rows_k, float scale2 /* scale * log2(e) */, int causal)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -239,8 +240,14 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
 #pragma unroll
                 for (int i = 0; i < 16; ++i) oacc[t][i] += op[(t * 16 + i) * WAVE + l] * f;
         }
+        m = M;                                   // the sums are relative to the team's reference point now
     }
     const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+    // log2 of the row's sum of exponentials of the scaled scores (what the backward pass needs to
+    // rebuild the probabilities); +inf for a row that sees nothing, so that they come out as zeros
+    if (lse != nullptr && h == 0)
+        lse[(size_t)batch * rows_q + BS * r + qq] = lsum > 0.f ? at_finite_or_zero(m) + __builtin_amdgcn_logf(lsum)
+                                                               : __builtin_inff();
     half_t *orow = out + ((size_t)batch * rows_q + BS * r + qq) * AT_HEAD + 4 * h;
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
@@ -254,10 +261,154 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Backward, first half: the probabilities P and the score gradients dS of every stored block in one
+// launch, from q, k, v, dO, O and the row statistics of the forward pass:
+//   P  = exp2(scale2 * q k^T - lse)                         (no second softmax pass: lse is known)
+//   dS = scale * P o (dO v^T - delta),  delta_q = sum_d dO_qd O_qd
+// This replaces SDD(q, k), softmax forward, SDD(dO, v) and softmax backward of the unfused chain
+// (four launches, 350 MB of score traffic at seq 4096) by one kernel that only WRITES the two block
+// stacks.  Same walk as the forward kernel (a lane holds one query column of S^T and dP^T), but the
+// blocks are independent of each other, so no running maximum, no merge.  The three products that
+// follow (dq = dS k, dk = dS^T q, dv = P^T dO) are DSD launches on P and dS.
+// ---------------------------------------------------------------------------
+constexpr int at_bwd_lds_per_wave(int hd) { return 128 * hd; }      // K tiles + V tiles, [key][32 d] each
+
+template <int HD, bool BF>
+__global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
+    const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
+    const half_t *__restrict__ dout, const half_t *__restrict__ out, const float *__restrict__ lse,
+    half_t *__restrict__ p_out, half_t *__restrict__ ds_out,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int rows_q, int rows_k, int nnz, float scale, int causal)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    if (e.group < 0 || e.begin >= e.end) return;
+    const int r = e.group;
+    const int qq = l & 31, h = l >> 5;
+    constexpr int KT = HD / 32;
+    const float scale2 = scale * 1.4426950408889634f;
+
+    half_t *tile_k = reinterpret_cast<half_t *>(lds_raw + (size_t)w * at_bwd_lds_per_wave(HD));
+    half_t *tile_v = tile_k + KT * BS2;
+    const half_t *kb = k + (size_t)batch * rows_k * HD;
+    const half_t *vb = v + (size_t)batch * rows_k * HD;
+    half_t *pb = p_out + (size_t)batch * nnz * BS2;
+    half_t *dsb = ds_out + (size_t)batch * nnz * BS2;
+
+    // column operands of the two products: lane (qq, h) holds d = 16 s + 8 h .. + 7 of query qq
+    const size_t qoff = ((size_t)batch * rows_q + BS * r + qq) * HD + 8 * h;
+    h8 qop[HD / 16], dop[HD / 16];
+    float delta = 0.f;
+#pragma unroll
+    for (int s = 0; s < HD / 16; ++s) {
+        qop[s] = as_h8(ldg16(q + qoff + 16 * s));
+        dop[s] = as_h8(ldg16(dout + qoff + 16 * s));
+        const h8 o = as_h8(ldg16(out + qoff + 16 * s));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) delta += widen_16<BF>(dop[s][i]) * widen_16<BF>(o[i]);
+    }
+    delta += at_lane_xor32(delta);               // the other half of the head dim sits in lane l ^ 32
+    const float row_lse = lse[(size_t)batch * rows_q + BS * r + qq];
+
+    struct Frag { uint4 kk[KT][2], vv[KT][2]; };
+    DescWindow win;
+    auto load = [&](int p, Frag &f) {
+        const int c = win.get(p).col();
+#pragma unroll
+        for (int dt = 0; dt < KT; ++dt) {
+            ldg_tile32(kb + (size_t)(BS * c) * HD + 32 * dt, HD, f.kk[dt]);
+            ldg_tile32(vb + (size_t)(BS * c) * HD + 32 * dt, HD, f.vv[dt]);
+        }
+    };
+    Frag fr;
+    for (int seg = e.begin; seg < e.end; seg += WAVE) {
+        const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+        win.fetch(blocks, seg, seg_end);
+        load(seg, fr);
+        for (int p = seg; p < seg_end; ++p) {
+            const BlockDesc d = win.get(p);
+            const int c = d.col();
+            wave_lds_fence();
+#pragma unroll
+            for (int dt = 0; dt < KT; ++dt) {
+                lds_put_kc<false>(tile_k + dt * BS2, fr.kk[dt]);
+                lds_put_kc<false>(tile_v + dt * BS2, fr.vv[dt]);
+            }
+            wave_lds_fence();
+            if (p + 1 < seg_end) load(p + 1, fr);
+            f16v sacc = {0}, dpacc = {0};
+#pragma unroll
+            for (int dt = 0; dt < KT; ++dt)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    sacc = mfma_16<BF>(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
+                    dpacc = mfma_16<BF>(lds_get_kc(tile_v + dt * BS2, s), dop[2 * dt + s], dpacc);
+                }
+            // Accumulator value i of lane half h is key 8 (i / 4) + 4 h + i % 4 of query qq: four runs of 4
+            // keys.  Written from here a store instruction would touch 64 separate 8-byte pieces, so
+            // the two result blocks go through the (now idle) staging tiles and leave as whole 2 KB
+            // pieces, like the SDD result.
+            wave_lds_fence();
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                h4 pv, dv;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = 4 * g + j, key = 8 * g + 4 * h + j;
+                    float pr = at_exp2(__builtin_fmaf(sacc[i], scale2, -row_lse));
+                    if (causal && (c > r || (c == r && key > qq))) pr = 0.f;
+                    pv[j] = narrow_16<BF>(pr);
+                    dv[j] = narrow_16<BF>(scale * pr * (dpacc[i] - delta));
+                }
+                const int at = 16 * kc_slot(qq, g) + 8 * h;       // 16-byte piece g of row qq, its half h
+                *reinterpret_cast<h4 *>(lds_bytes(tile_k) + at) = pv;
+                *reinterpret_cast<h4 *>(lds_bytes(tile_v) + at) = dv;
+            }
+            wave_lds_fence();
+            uint4 raw[2];
+            lds_get_linear(tile_k, raw);
+            stg_tile32(pb + (size_t)d.idx * BS2, raw);
+            lds_get_linear(tile_v, raw);
+            stg_tile32(dsb + (size_t)d.idx * BS2, raw);
+        }
+    }
+}
+
+hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t st)
+{
+    dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
+    const size_t lds = (size_t)p.sched_waves * at_bwd_lds_per_wave(p.head_dim);
+#define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (const half_t *)p.dout, \
+                    (const half_t *)p.out, (const float *)p.lse, (half_t *)p.p_out, (half_t *)p.ds_out, \
+                    (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
+                    32 * p.mask_rows, 32 * p.mask_cols, p.nnz, p.scale, p.causal ? 1 : 0
+    if (p.head_dim == 64) {
+        if (p.bf16) attention_bwd_scores_kernel<64, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+        else attention_bwd_scores_kernel<64, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+    } else {
+        if (lds > 65536) {
+            const void *fn = p.bf16 ? (const void *)attention_bwd_scores_kernel<128, true>
+                                    : (const void *)attention_bwd_scores_kernel<128, false>;
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        if (p.bf16) attention_bwd_scores_kernel<128, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+        else attention_bwd_scores_kernel<128, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+    }
+#undef BSA_AT_ARGS
+    return hipGetLastError();
+}
+
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t st)
 {
     dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
-#define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (half_t *)p.out, \
+#define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (half_t *)p.out, (float *)p.lse, \
                     (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
                     32 * p.mask_rows, 32 * p.mask_cols, p.scale * 1.4426950408889634f, p.causal ? 1 : 0
     const size_t lds = (size_t)p.sched_waves * at_lds_per_wave(p.head_dim);

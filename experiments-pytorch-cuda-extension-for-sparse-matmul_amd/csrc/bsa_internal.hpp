@@ -58,7 +58,11 @@ hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t 
 
 struct AttentionArgs {
     const void *q, *k, *v;
-    void *out;
+    void *out;              // forward: result; backward: the forward result (read)
+    void *lse;              // forward: optional output; backward: input
+    const void *dout;       // backward only
+    void *p_out, *ds_out;   // backward only: [batches, nnz, 32, 32] each
+    int nnz;
     const int32_t *blocks;
     const int32_t *sched;
     int groups;
@@ -71,5 +75,6 @@ struct AttentionArgs {
 };
 
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t stream);
+hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t stream);
 
 }  // namespace bsa

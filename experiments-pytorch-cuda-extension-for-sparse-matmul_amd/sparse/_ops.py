@@ -17,6 +17,7 @@ GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
 SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
+SCHEDULE_ATTENTION_BACKWARD = (4, 2)  # P / dS kernel: blocks are independent, short chunks
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
@@ -233,10 +234,7 @@ def sparse_softmax_backward(y, dy, row_blocks, row_table, scale=1.0, col_layout=
     return dx
 
 
-def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=False, col_layout=None):
-    """``softmax(scale * q k^T on the stored blocks) v`` in one launch: the chain of
-    ``sparse_matmul('sdd', trans_b)``, the softmax and ``sparse_matmul('dsd')`` (sparse/matmul.py:57,
-    sparse_softmax.cu:208-231) without the scores in memory.  fp16 / bf16, head dim 64 or 128."""
+def _attention_common(q, k, v, row_blocks, row_table, col_layout):
     row_layout = (row_blocks, row_table)
     _check_layout(row_layout, "row_layout")
     for t, name in ((q, "q"), (k, "k"), (v, "v")):
@@ -248,26 +246,63 @@ def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=F
             raise ValueError(f"{name} needs at least one batch dimension, got shape {tuple(t.shape)}")
     if row_blocks.device != q.device:
         raise ValueError("layout tables and operands must live on the same GPU")
-    mask_rows = row_table.numel() - 1
     if col_layout is None:
         raise ValueError("col_layout is needed for the number of block columns")
-    mask_cols = col_layout[1].numel() - 1
-    nnz = row_blocks.numel() // 2
+    mask_rows, mask_cols = row_table.numel() - 1, col_layout[1].numel() - 1
     head = q.size(-1)
     if q.size(-2) != mask_rows * BLOCK or k.size(-2) != mask_cols * BLOCK or k.shape != v.shape \
             or k.size(-1) != head or q.shape[:-2] != k.shape[:-2]:
         raise ValueError(f"q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit a "
                          f"{mask_rows} x {mask_cols} block layout")
+    batches = q.numel() // max(q.size(-1) * q.size(-2), 1)
+    return row_layout, mask_rows, mask_cols, row_blocks.numel() // 2, head, batches
+
+
+def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=False, col_layout=None,
+                             return_lse=False):
+    """``softmax(scale * q k^T on the stored blocks) v`` in one launch: the chain of
+    ``sparse_matmul('sdd', trans_b)``, the softmax and ``sparse_matmul('dsd')`` (sparse/matmul.py:57,
+    sparse_softmax.cu:208-231) without the scores in memory.  fp16 / bf16, head dim 64 or 128.
+    With ``return_lse`` also the fp32 row statistics the backward pass needs."""
+    row_layout, mask_rows, mask_cols, nnz, head, batches = _attention_common(q, k, v, row_blocks, row_table,
+                                                                              col_layout)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     out = torch.empty_like(q)
-    if out.numel() == 0:
-        return out
-    batches = q.numel() // (q.size(-1) * q.size(-2))
-    cap, waves = SCHEDULE_ATTENTION
-    sched = schedule_for(row_layout, (cap, waves, False))
-    with torch.cuda.device(q.device):
-        _k.check(_k.lib.bsa_attention_forward(
-            _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-            row_blocks.data_ptr(), row_table.data_ptr(), sched.table.data_ptr(), sched.workgroups, sched.waves,
-            mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), _k.current_stream()))
-    return out
+    lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device) if return_lse else None
+    if out.numel() > 0:
+        cap, waves = SCHEDULE_ATTENTION
+        sched = schedule_for(row_layout, (cap, waves, False))
+        with torch.cuda.device(q.device):
+            _k.check(_k.lib.bsa_attention_forward(
+                _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                lse.data_ptr() if lse is not None else None,
+                row_blocks.data_ptr(), row_table.data_ptr(), sched.table.data_ptr(), sched.workgroups, sched.waves,
+                mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), _k.current_stream()))
+    return (out, lse) if return_lse else out
+
+
+def sparse_attention_backward_scores(q, k, v, dout, out, lse, row_blocks, row_table, scale=1.0, causal=False,
+                                     col_layout=None):
+    """Probabilities and score gradients of every stored block, ``[..., nnz, 32, 32]`` each, in one
+    launch: what ``sparse_matmul('sdd')``, the softmax forward, ``sparse_matmul('sdd')`` on ``dout, v``
+    and the softmax backward (sparse_softmax.cu:165-205) give with four."""
+    row_layout, mask_rows, mask_cols, nnz, head, batches = _attention_common(q, k, v, row_blocks, row_table,
+                                                                              col_layout)
+    if dout.shape != q.shape or out.shape != q.shape or dout.dtype != q.dtype or out.dtype != q.dtype:
+        raise ValueError("dout and out must match q in shape and dtype")
+    if lse.dtype != torch.float32 or lse.shape != q.shape[:-1]:
+        raise ValueError("lse must be the float32 row statistics of the forward pass")
+    q, k, v, dout, out, lse = (t.contiguous() for t in (q, k, v, dout, out, lse))
+    shape = q.shape[:-2] + (nnz, BLOCK, BLOCK)
+    p = torch.empty(shape, dtype=q.dtype, device=q.device)
+    ds = torch.empty(shape, dtype=q.dtype, device=q.device)
+    if p.numel() > 0:
+        cap, waves = SCHEDULE_ATTENTION_BACKWARD
+        sched = schedule_for(row_layout, (cap, waves, False))
+        with torch.cuda.device(q.device):
+            _k.check(_k.lib.bsa_attention_backward_scores(
+                _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
+                lse.data_ptr(), p.data_ptr(), ds.data_ptr(), row_blocks.data_ptr(), row_table.data_ptr(),
+                sched.table.data_ptr(), sched.workgroups, sched.waves, mask_rows, mask_cols, nnz, batches, head,
+                float(scale), int(bool(causal)), _k.current_stream()))
+    return p, ds

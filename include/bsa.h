@@ -191,15 +191,34 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
  * in a row; the probabilities are rounded to fp16 before the second product, as there.
  *   q    [batches, 32 * mask_rows, head_dim], k, v  [batches, 32 * mask_cols, head_dim], contiguous
  *   out  [batches, 32 * mask_rows, head_dim]; rows without stored (or unmasked) blocks give zeros
+ *   lse  optional (may be NULL) float[batches, 32 * mask_rows]: log2 of every row's sum of
+ *        2^(scale * log2(e) * score); +inf for a row that sees nothing.  The backward pass needs it.
  *   tables / schedule: those of the ROW layout; the schedule must be built with
  *   allow_split = 0 and slice_max = -1 (a block row stays inside one workgroup).
  * fp16 and bf16 only, head_dim 64 or 128 (BSA_ERR_UNSUPPORTED otherwise).
  */
-int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out,
+int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out, float *lse,
                           const int32_t *row_blocks, const int32_t *row_offsets,
                           const int32_t *sched, int sched_wgs, int sched_waves,
                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                           float scale, int causal, void *stream);
+
+/* First half of the attention backward pass in one launch: from q, k, v, the gradient `dout` of the
+ * result, the forward result `out` and `lse`, the probabilities and the score gradients of every
+ * stored block,
+ *   p_out  = softmax probabilities                         [batches, nnz, 32, 32]
+ *   ds_out = scale * p o (dout v^T - rowsum(dout o out))   [batches, nnz, 32, 32]
+ * i.e. what SDD(q, k), the softmax forward, SDD(dout, v) and the softmax backward of the unfused
+ * chain produce with four launches (sparse_smm_gpu.cu:22-95 twice, sparse_softmax.cu:113-205).
+ * The caller finishes with three DSD products: dq = ds k, dk = ds^T q, dv = p^T dout.
+ * Same tables, schedule (any row schedule: blocks are independent here) and limits as the forward.
+ */
+int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const void *v, const void *dout,
+                                  const void *out, const float *lse, void *p_out, void *ds_out,
+                                  const int32_t *row_blocks, const int32_t *row_offsets,
+                                  const int32_t *sched, int sched_wgs, int sched_waves,
+                                  int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
+                                  float scale, int causal, void *stream);
 
 #ifdef __cplusplus
 }

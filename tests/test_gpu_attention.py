@@ -117,3 +117,44 @@ def test_argument_checks():
         sparse.attention(q[:, :64], k, v, L)
     with pytest.raises(Exception):
         sparse.attention(q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous(), L)   # head dim 32
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("name,head", [("known3x3", 64), ("rand16", 64), ("long_row_5x40", 64), ("empty_row_col_6x5", 128)])
+def test_row_statistics_and_backward_scores(name, head, causal):
+    """lse of the forward kernel, and P / dS of the one-launch backward half, against float64."""
+    from sparse.kernel import sparse_ops
+    from oracle import layout_oracle as lo
+    import sparse
+    mask = np.asarray(ZOO[name])
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    q, k, v = _qkv(mask, seed=17, head=head)
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(18)).half()
+    scale = 0.11
+    rows, cols = L.row_layout, L.col_layout
+    out, lse = sparse_ops.sparse_attention_forward(q.cuda(), k.cuda(), v.cuda(), rows[0], rows[1], scale, causal,
+                                                   cols, return_lse=True)
+    # float64 reference of the dense meaning
+    vis = np.repeat(np.repeat(mask != 0, 32, 0), 32, 1)
+    if causal:
+        r_, c_ = np.indices(vis.shape)
+        vis &= c_ <= r_
+    s = scale * np.einsum("bqd,bkd->bqk", to_np(q), to_np(k))
+    s = np.where(vis, s, -np.inf)
+    with np.errstate(divide="ignore"):
+        ref_lse = np.log2(np.sum(np.exp(s - np.where(np.isfinite(s.max(-1, keepdims=True)), s.max(-1, keepdims=True), 0)), -1)) \
+                  + np.where(np.isfinite(s.max(-1)), s.max(-1), 0) * np.log2(np.e)
+    seen = vis.any(axis=1)
+    got = to_np(lse)
+    assert np.all(np.isposinf(got[:, ~seen]))
+    assert np.max(np.abs(got[:, seen] - ref_lse[:, seen])) <= 2e-3 * max(1.0, np.max(np.abs(ref_lse[:, seen])))
+    p, ds = sparse_ops.sparse_attention_backward_scores(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), out, lse,
+                                                        rows[0], rows[1], scale, causal, cols)
+    pd = np.exp(s - np.where(np.isfinite(s.max(-1, keepdims=True)), s.max(-1, keepdims=True), 0))
+    den = pd.sum(-1, keepdims=True)
+    pd = np.divide(pd, den, out=np.zeros_like(pd), where=den > 0)
+    dp = np.einsum("bqd,bkd->bqk", to_np(dout), to_np(v))
+    delta = np.sum(to_np(dout) * (pd @ to_np(v)), -1, keepdims=True)
+    dsd = scale * pd * (dp - delta)
+    assert rel_err(to_np(p), lo.to_sparse(mask, pd)) <= TOL
+    assert rel_err(to_np(ds), lo.to_sparse(mask, dsd)) <= 2 * TOL
