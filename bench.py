@@ -175,7 +175,7 @@ def main():
         attention[name + "_nnz_TFLOPs"] = round(2 * flops_one / (ms * 1e-3) / 1e12, 2)
     attention["speedup"] = round(attention["chain_us"] / attention["fused_us"], 2)
 
-    # the backward pass of the same attention: one launch for P and dS + three products, against the
+    # the backward pass of the same attention: one launch for P, dS and dq + two products, against the
     # seven launches of the unfused chain (gradients of q, k, v from dout)
     from sparse.kernel import sparse_ops
     rows, cols = layout.row_layout, layout.col_layout
@@ -184,14 +184,15 @@ def main():
         w["out"], w["lse"] = sparse_ops.sparse_attention_forward(w["q"], w["k"], w["v"], rows[0], rows[1], 0.125, True,
                                                                  cols, return_lse=True)
 
-    def products(p, ds, w):
-        return (sparse.matmul(ds, w["k"], "dsd", layout), sparse.matmul(ds, w["q"], "dsd", layout, True, False),
+    def products(p, ds, w, with_dq=True):
+        return (sparse.matmul(ds, w["k"], "dsd", layout) if with_dq else None,
+                sparse.matmul(ds, w["q"], "dsd", layout, True, False),
                 sparse.matmul(p, w["dout"], "dsd", layout, True, False))
 
     def backward_fused(w):
-        p, ds = sparse_ops.sparse_attention_backward_scores(w["q"], w["k"], w["v"], w["dout"], w["out"], w["lse"],
-                                                            rows[0], rows[1], 0.125, True, cols)
-        return products(p, ds, w)
+        p, ds, dq = sparse_ops.sparse_attention_backward_scores(w["q"], w["k"], w["v"], w["dout"], w["out"], w["lse"],
+                                                                rows[0], rows[1], 0.125, True, cols)
+        return (dq,) + products(p, ds, w, with_dq=False)[1:]
 
     def backward_chain(w):
         p = sparse.softmax(sparse.matmul(w["q"], w["k"], "sdd", layout, False, True), layout, 0.125, True)

@@ -286,14 +286,14 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
                              mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
     if (!q || !k || !v || !out) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
-    bsa::AttentionArgs p{q, k, v, out, lse, nullptr, nullptr, nullptr, nnz, row_blocks, sched, mask_rows,
+    bsa::AttentionArgs p{q, k, v, out, lse, nullptr, nullptr, nullptr, nullptr, nnz, row_blocks, sched, mask_rows,
                          sched_wgs, sched_waves, mask_rows, mask_cols, batches, scale, causal != 0,
                          dtype == BSA_BF16, head_dim};
     return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
 }
 
 int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const void *v, const void *dout,
-                                  const void *out, const float *lse, void *p_out, void *ds_out,
+                                  const void *out, const float *lse, void *p_out, void *ds_out, void *dq_out,
                                   const int32_t *row_blocks, const int32_t *row_offsets,
                                   const int32_t *sched, int sched_wgs, int sched_waves,
                                   int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
@@ -303,10 +303,10 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
     int rc = check_attention(who, dtype, head_dim, row_blocks, row_offsets, sched, sched_wgs, sched_waves,
                              mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
-    if (nnz == 0) return BSA_OK;      // no blocks to write
-    if (!q || !k || !v || !dout || !out || !lse || !p_out || !ds_out)
+    if (nnz == 0 && !dq_out) return BSA_OK;      // no blocks to write
+    if (!q || !k || !v || !dout || !out || !lse || (nnz > 0 && (!p_out || !ds_out)))
         return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
-    bsa::AttentionArgs p{q, k, v, const_cast<void *>(out), const_cast<float *>(lse), dout, p_out, ds_out, nnz,
+    bsa::AttentionArgs p{q, k, v, const_cast<void *>(out), const_cast<float *>(lse), dout, p_out, ds_out, dq_out, nnz,
                          row_blocks, sched, mask_rows, sched_wgs, sched_waves, mask_rows, mask_cols, batches,
                          scale, causal != 0, dtype == BSA_BF16, head_dim};
     return check_launch(bsa::launch_attention_backward_scores(p, (hipStream_t)stream), who);

@@ -262,23 +262,29 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Backward, first half: the probabilities P and the score gradients dS of every stored block in one
-// launch, from q, k, v, dO, O and the row statistics of the forward pass:
+// Backward, first half: the probabilities P and the score gradients dS of every stored block, and
+// dq, in one launch, from q, k, v, dO, O and the row statistics of the forward pass:
 //   P  = exp2(scale2 * q k^T - lse)                         (no second softmax pass: lse is known)
 //   dS = scale * P o (dO v^T - delta),  delta_q = sum_d dO_qd O_qd
-// This replaces SDD(q, k), softmax forward, SDD(dO, v) and softmax backward of the unfused chain
-// (four launches, 350 MB of score traffic at seq 4096) by one kernel that only WRITES the two block
-// stacks.  Same walk as the forward kernel (a lane holds one query column of S^T and dP^T), but the
-// blocks are independent of each other, so no running maximum, no merge.  The three products that
-// follow (dq = dS k, dk = dS^T q, dv = P^T dO) are DSD launches on P and dS.
+//   dq^T += K_c^T dS^T                                       (K_c is on the chip already)
+// This replaces SDD(q, k), softmax forward, SDD(dO, v), softmax backward and the DSD product dS k
+// of the unfused chain (five launches, 350 MB of score traffic at seq 4096 and dS read once more) by
+// one kernel that only WRITES the two block stacks.  Same walk as the forward kernel: a lane holds
+// one query column of S^T and dP^T, and the fp16 dS values feed the dq product straight from those
+// registers (the K_c tiles are read a second time along their rows, the reader exchanging rows the way
+// the forward kernel parks V_c).
+// The waves of a row add their dq^T parts through LDS.  The two products that follow
+// (dk = dS^T q, dv = P^T dO) walk the columns and are DSD launches on P and dS.
 // ---------------------------------------------------------------------------
-constexpr int at_bwd_lds_per_wave(int hd) { return 128 * hd; }      // K tiles + V tiles, [key][32 d] each
+// per wave: K tiles + V tiles, [key][32 d] each; the V tiles take the two result blocks afterwards, and
+// the whole the dq^T part of the merge (HD x 32 floats)
+constexpr int at_bwd_lds_per_wave(int hd) { return 128 * hd; }
 
 template <int HD, bool BF>
 __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
     const half_t *__restrict__ dout, const half_t *__restrict__ out, const float *__restrict__ lse,
-    half_t *__restrict__ p_out, half_t *__restrict__ ds_out,
+    half_t *__restrict__ p_out, half_t *__restrict__ ds_out, half_t *__restrict__ dq_out,
     const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
     int n_swg, int batches, int rows_q, int rows_k, int nnz, float scale, int causal)
 {
@@ -288,96 +294,144 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
     const int w = wave_id(), l = lane_id();
     const int W = (int)(blockDim.x >> 6);
     const SchedEntry e = sched[swg * W + w];
-    if (e.group < 0 || e.begin >= e.end) return;
+    const bool active = e.group >= 0;
     const int r = e.group;
     const int qq = l & 31, h = l >> 5;
-    constexpr int KT = HD / 32;
+    constexpr int KT = HD / 32, LDS_PER_WAVE = at_bwd_lds_per_wave(HD);
     const float scale2 = scale * 1.4426950408889634f;
 
-    half_t *tile_k = reinterpret_cast<half_t *>(lds_raw + (size_t)w * at_bwd_lds_per_wave(HD));
+    unsigned char *my_lds = lds_raw + (size_t)w * LDS_PER_WAVE;
+    half_t *tile_k = reinterpret_cast<half_t *>(my_lds);
     half_t *tile_v = tile_k + KT * BS2;
     const half_t *kb = k + (size_t)batch * rows_k * HD;
     const half_t *vb = v + (size_t)batch * rows_k * HD;
     half_t *pb = p_out + (size_t)batch * nnz * BS2;
     half_t *dsb = ds_out + (size_t)batch * nnz * BS2;
 
-    // column operands of the two products: lane (qq, h) holds d = 16 s + 8 h .. + 7 of query qq
-    const size_t qoff = ((size_t)batch * rows_q + BS * r + qq) * HD + 8 * h;
-    h8 qop[HD / 16], dop[HD / 16];
-    float delta = 0.f;
+    f16v dqacc[KT];                              // dq^T: lane = query column, values = head dims as in the forward kernel
 #pragma unroll
-    for (int s = 0; s < HD / 16; ++s) {
-        qop[s] = as_h8(ldg16(q + qoff + 16 * s));
-        dop[s] = as_h8(ldg16(dout + qoff + 16 * s));
-        const h8 o = as_h8(ldg16(out + qoff + 16 * s));
-#pragma unroll
-        for (int i = 0; i < 8; ++i) delta += widen_16<BF>(dop[s][i]) * widen_16<BF>(o[i]);
-    }
-    delta += at_lane_xor32(delta);               // the other half of the head dim sits in lane l ^ 32
-    const float row_lse = lse[(size_t)batch * rows_q + BS * r + qq];
+    for (int t = 0; t < KT; ++t) dqacc[t] = f16v{0};
 
-    struct Frag { uint4 kk[KT][2], vv[KT][2]; };
-    DescWindow win;
-    auto load = [&](int p, Frag &f) {
-        const int c = win.get(p).col();
+    if (active && e.begin < e.end) {
+        // column operands of the two products: lane (qq, h) holds d = 16 s + 8 h .. + 7 of query qq
+        const size_t qoff = ((size_t)batch * rows_q + BS * r + qq) * HD + 8 * h;
+        h8 qop[HD / 16], dop[HD / 16];
+        float delta = 0.f;
 #pragma unroll
-        for (int dt = 0; dt < KT; ++dt) {
-            ldg_tile32(kb + (size_t)(BS * c) * HD + 32 * dt, HD, f.kk[dt]);
-            ldg_tile32(vb + (size_t)(BS * c) * HD + 32 * dt, HD, f.vv[dt]);
+        for (int s = 0; s < HD / 16; ++s) {
+            qop[s] = as_h8(ldg16(q + qoff + 16 * s));
+            dop[s] = as_h8(ldg16(dout + qoff + 16 * s));
+            const h8 o = as_h8(ldg16(out + qoff + 16 * s));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) delta += widen_16<BF>(dop[s][i]) * widen_16<BF>(o[i]);
         }
-    };
-    Frag fr;
-    for (int seg = e.begin; seg < e.end; seg += WAVE) {
-        const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
-        win.fetch(blocks, seg, seg_end);
-        load(seg, fr);
-        for (int p = seg; p < seg_end; ++p) {
-            const BlockDesc d = win.get(p);
-            const int c = d.col();
-            wave_lds_fence();
+        delta += at_lane_xor32(delta);           // the other half of the head dim sits in lane l ^ 32
+        const float row_lse = lse[(size_t)batch * rows_q + BS * r + qq];
+
+        struct Frag { uint4 kk[KT][2], vv[KT][2]; };
+        DescWindow win;
+        auto load = [&](int p, Frag &f) {
+            const int c = win.get(p).col();
 #pragma unroll
             for (int dt = 0; dt < KT; ++dt) {
-                lds_put_kc<false>(tile_k + dt * BS2, fr.kk[dt]);
-                lds_put_kc<false>(tile_v + dt * BS2, fr.vv[dt]);
+                ldg_tile32(kb + (size_t)(BS * c) * HD + 32 * dt, HD, f.kk[dt]);
+                ldg_tile32(vb + (size_t)(BS * c) * HD + 32 * dt, HD, f.vv[dt]);
             }
-            wave_lds_fence();
-            if (p + 1 < seg_end) load(p + 1, fr);
-            f16v sacc = {0}, dpacc = {0};
+        };
+        Frag fr;
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+            load(seg, fr);
+            for (int p = seg; p < seg_end; ++p) {
+                const BlockDesc d = win.get(p);
+                const int c = d.col();
+                wave_lds_fence();
 #pragma unroll
-            for (int dt = 0; dt < KT; ++dt)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    sacc = mfma_16<BF>(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
-                    dpacc = mfma_16<BF>(lds_get_kc(tile_v + dt * BS2, s), dop[2 * dt + s], dpacc);
+                for (int dt = 0; dt < KT; ++dt) {
+                    lds_put_kc<false>(tile_k + dt * BS2, fr.kk[dt]);
+                    lds_put_kc<false>(tile_v + dt * BS2, fr.vv[dt]);
                 }
-            // Accumulator value i of lane half h is key 8 (i / 4) + 4 h + i % 4 of query qq: four runs of 4
-            // keys.  Written from here a store instruction would touch 64 separate 8-byte pieces, so
-            // the two result blocks go through the (now idle) staging tiles and leave as whole 2 KB
-            // pieces, like the SDD result.
-            wave_lds_fence();
+                wave_lds_fence();
+                if (p + 1 < seg_end) load(p + 1, fr);
+                f16v sacc = {0}, dpacc = {0};
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                h4 pv, dv;
+                for (int dt = 0; dt < KT; ++dt)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int i = 4 * g + j, key = 8 * g + 4 * h + j;
-                    float pr = at_exp2(__builtin_fmaf(sacc[i], scale2, -row_lse));
-                    if (causal && (c > r || (c == r && key > qq))) pr = 0.f;
-                    pv[j] = narrow_16<BF>(pr);
-                    dv[j] = narrow_16<BF>(scale * pr * (dpacc[i] - delta));
+                    for (int s = 0; s < 2; ++s) {
+                        sacc = mfma_16<BF>(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
+                        dpacc = mfma_16<BF>(lds_get_kc(tile_v + dt * BS2, s), dop[2 * dt + s], dpacc);
+                    }
+                // Accumulator value i of lane half h is key 8 (i / 4) + 4 h + i % 4 of query qq: four runs of 4
+                // keys.  Written from here a store instruction would touch 64 separate 8-byte pieces, so
+                // the two result blocks go through the (now idle) V tiles and leave as whole 2 KB
+                // pieces, like the SDD result.  The K tiles stay: dq reads them once more.
+                wave_lds_fence();
+                h8 dsop[2];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    h4 pv, dv;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int i = 4 * g + j, key = 8 * g + 4 * h + j;
+                        float pr = at_exp2(__builtin_fmaf(sacc[i], scale2, -row_lse));
+                        if (causal && (c > r || (c == r && key > qq))) pr = 0.f;
+                        pv[j] = narrow_16<BF>(pr);
+                        dv[j] = narrow_16<BF>(scale * pr * (dpacc[i] - delta));
+                        dsop[i >> 3][i & 7] = dv[j];
+                    }
+                    const int at = 16 * kc_slot(qq, g) + 8 * h;       // 16-byte piece g of row qq, its half h
+                    *reinterpret_cast<h4 *>(lds_bytes(tile_v) + at) = pv;
+                    *reinterpret_cast<h4 *>(lds_bytes(tile_v + BS2) + at) = dv;
                 }
-                const int at = 16 * kc_slot(qq, g) + 8 * h;       // 16-byte piece g of row qq, its half h
-                *reinterpret_cast<h4 *>(lds_bytes(tile_k) + at) = pv;
-                *reinterpret_cast<h4 *>(lds_bytes(tile_v) + at) = dv;
+                if (dq_out != nullptr) {
+#pragma unroll
+                    for (int t = 0; t < KT; ++t)
+#pragma unroll
+                        for (int s = 0; s < 2; ++s)
+                            dqacc[t] = mfma_16<BF>(lds_get_kc_tr_swapped(tile_k + t * BS2, s), dsop[s], dqacc[t]);
+                }
+                wave_lds_fence();
+                uint4 raw[2];
+                lds_get_linear(tile_v, raw);
+                stg_tile32(pb + (size_t)d.idx * BS2, raw);
+                lds_get_linear(tile_v + BS2, raw);
+                stg_tile32(dsb + (size_t)d.idx * BS2, raw);
             }
-            wave_lds_fence();
-            uint4 raw[2];
-            lds_get_linear(tile_k, raw);
-            stg_tile32(pb + (size_t)d.idx * BS2, raw);
-            lds_get_linear(tile_v, raw);
-            stg_tile32(dsb + (size_t)d.idx * BS2, raw);
         }
     }
+    if (dq_out == nullptr) return;               // uniform over the launch
+
+    // team merge: every wave of a row but the leader parks its dq^T part, the leader adds and stores
+    const int slot0 = e.first_wave(), nw = e.team_waves();
+    const bool leader = active && w == slot0;
+    float *park = reinterpret_cast<float *>(my_lds);
+    if (active && !leader) {
+        wave_lds_fence();
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) park[(t * 16 + i) * WAVE + l] = dqacc[t][i];
+    }
+    __syncthreads();
+    if (!leader) return;
+    for (int o = 1; o < nw; ++o) {
+        const float *op = reinterpret_cast<const float *>(lds_raw + (size_t)(w + o) * LDS_PER_WAVE);
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dqacc[t][i] += op[(t * 16 + i) * WAVE + l];
+    }
+    half_t *drow = dq_out + ((size_t)batch * rows_q + BS * r + qq) * HD + 4 * h;
+#pragma unroll
+    for (int t = 0; t < KT; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            h4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = narrow_16<BF>(dqacc[t][4 * g + j]);
+            *reinterpret_cast<h4 *>(drow + 32 * t + 8 * g) = o;
+        }
 }
 
 hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t st)
@@ -385,7 +439,7 @@ hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t 
     dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
     const size_t lds = (size_t)p.sched_waves * at_bwd_lds_per_wave(p.head_dim);
 #define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (const half_t *)p.dout, \
-                    (const half_t *)p.out, (const float *)p.lse, (half_t *)p.p_out, (half_t *)p.ds_out, \
+                    (const half_t *)p.out, (const float *)p.lse, (half_t *)p.p_out, (half_t *)p.ds_out, (half_t *)p.dq_out, \
                     (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
                     32 * p.mask_rows, 32 * p.mask_cols, p.nnz, p.scale, p.causal ? 1 : 0
     if (p.head_dim == 64) {

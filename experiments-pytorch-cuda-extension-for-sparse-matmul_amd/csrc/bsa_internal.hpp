@@ -62,6 +62,7 @@ struct AttentionArgs {
     void *lse;              // forward: optional output; backward: input
     const void *dout;       // backward only
     void *p_out, *ds_out;   // backward only: [batches, nnz, 32, 32] each
+    void *dq_out;           // backward only, may be null: [batches, 32 mask_rows, head_dim]
     int nnz;
     const int32_t *blocks;
     const int32_t *sched;

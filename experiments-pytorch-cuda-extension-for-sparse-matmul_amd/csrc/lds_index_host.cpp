@@ -16,6 +16,7 @@ extern "C" int bsa_lds_access(const char *name, int permuted, int arg0, int arg1
         else if (!strcmp(name, "get_ks")) a = get_ks_addr(permuted, lane, arg0, arg1);
         else if (!strcmp(name, "put_strip")) a = put_strip_addr(lane, arg0);
         else if (!strcmp(name, "put_strip_swapped")) a = put_strip_swapped_addr(lane, arg0);
+        else if (!strcmp(name, "get_kc_tr_swapped")) a = get_kc_tr_swapped_addr(lane, arg0, arg1);
         else if (!strcmp(name, "get_strip")) a = get_strip_addr(permuted, lane, arg0 & 1, arg0 >> 1, arg1);
         else if (!strcmp(name, "put_result")) a = put_result_addr(lane, arg0);
         else if (!strcmp(name, "get_linear")) a = get_linear_addr(lane, arg0);

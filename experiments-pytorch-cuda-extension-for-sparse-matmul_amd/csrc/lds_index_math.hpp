@@ -91,6 +91,18 @@ BSA_HD constexpr int put_strip_swapped_addr(int lane, int q)
     int k = swap_bits23(c >> 3);
     return 16 * (k * 8 + ((c & 7) ^ strip_swizzle(k)));
 }
+// Transposing read of a [index][k] tile (the put_kc_addr layout, not permuted) along its ROWS: the
+// operand of a product that contracts over the tile's row index, with the same exchange of rows
+// 4-7 and 8-11 as above applied by the reader: element j of lane (index = lane % 32, h = lane / 32)
+// is row 16 step + 8 (j / 4) + 4 h + j % 4.  The 4 rows a 16-lane group touches share one
+// kc_swizzle and fill one 256-byte bank window.
+BSA_HD constexpr int get_kc_tr_swapped_addr(int lane, int step, int half)
+{
+    int g = lane >> 4, s = lane & 15;
+    int k = 16 * step + 4 * (g >> 1) + (s >> 2) + 8 * half;
+    int x = tr_chunk_base(false, g, s & 3) ^ (8 * kc_swizzle(k));
+    return 2 * (k * 32 + x);
+}
 BSA_HD constexpr int get_strip_addr(bool permuted, int lane, int step, int half, int x0)
 {
     int g = lane >> 4, s = lane & 15;

@@ -75,6 +75,15 @@ __device__ __forceinline__ h8 lds_get_ks(const half_t *tile, int step)
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// rows of a [index][k] tile as the contraction, rows 4-7 and 8-11 of every 16 exchanged (see get_kc_tr_swapped_addr)
+__device__ __forceinline__ h8 lds_get_kc_tr_swapped(const half_t *tile, int step)
+{
+    int l = lane_id();
+    h4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile) + get_kc_tr_swapped_addr(l, step, 0)));
+    h4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile) + get_kc_tr_swapped_addr(l, step, 1)));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // ---- [k][64] dense strip, 128-byte rows, XOR swizzle (group walk) -------------
 __device__ __forceinline__ void lds_put_strip(half_t *tile, const uint4 (&lo)[2], const uint4 (&hi)[2])
 {

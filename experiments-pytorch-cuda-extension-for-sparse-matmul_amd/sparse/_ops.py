@@ -17,7 +17,7 @@ GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
 SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
-SCHEDULE_ATTENTION_BACKWARD = (4, 2)  # P / dS kernel: blocks are independent, short chunks
+SCHEDULE_ATTENTION_BACKWARD = (16, 4)
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
@@ -282,10 +282,11 @@ def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=F
 
 
 def sparse_attention_backward_scores(q, k, v, dout, out, lse, row_blocks, row_table, scale=1.0, causal=False,
-                                     col_layout=None):
-    """Probabilities and score gradients of every stored block, ``[..., nnz, 32, 32]`` each, in one
-    launch: what ``sparse_matmul('sdd')``, the softmax forward, ``sparse_matmul('sdd')`` on ``dout, v``
-    and the softmax backward (sparse_softmax.cu:165-205) give with four."""
+                                     col_layout=None, with_dq=True):
+    """Probabilities and score gradients of every stored block, ``[..., nnz, 32, 32]`` each, and (with
+    ``with_dq``, else ``None``) the gradient of ``q``, in one launch: what ``sparse_matmul('sdd')``, the
+    softmax forward, ``sparse_matmul('sdd')`` on ``dout, v``, the softmax backward
+    (sparse_softmax.cu:165-205) and ``sparse_matmul('dsd')`` on ``ds, k`` give with five."""
     row_layout, mask_rows, mask_cols, nnz, head, batches = _attention_common(q, k, v, row_blocks, row_table,
                                                                               col_layout)
     if dout.shape != q.shape or out.shape != q.shape or dout.dtype != q.dtype or out.dtype != q.dtype:
@@ -296,13 +297,15 @@ def sparse_attention_backward_scores(q, k, v, dout, out, lse, row_blocks, row_ta
     shape = q.shape[:-2] + (nnz, BLOCK, BLOCK)
     p = torch.empty(shape, dtype=q.dtype, device=q.device)
     ds = torch.empty(shape, dtype=q.dtype, device=q.device)
-    if p.numel() > 0:
+    dq = torch.empty_like(q) if with_dq else None
+    if q.numel() > 0:
         cap, waves = SCHEDULE_ATTENTION_BACKWARD
         sched = schedule_for(row_layout, (cap, waves, False))
         with torch.cuda.device(q.device):
             _k.check(_k.lib.bsa_attention_backward_scores(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
-                lse.data_ptr(), p.data_ptr(), ds.data_ptr(), row_blocks.data_ptr(), row_table.data_ptr(),
+                lse.data_ptr(), p.data_ptr(), ds.data_ptr(), dq.data_ptr() if with_dq else None,
+                row_blocks.data_ptr(), row_table.data_ptr(),
                 sched.table.data_ptr(), sched.workgroups, sched.waves, mask_rows, mask_cols, nnz, batches, head,
                 float(scale), int(bool(causal)), _k.current_stream()))
-    return p, ds
+    return p, ds, dq

@@ -3,8 +3,8 @@
 The reference has no such call: its users chain ``matmul(q, k, 'sdd', layout, False, True)``, a
 softmax and ``matmul(p, v, 'dsd', layout)`` (``sparse/matmul.py:57``).  The forward here is ONE
 launch that keeps the scores on the chip; the backward rebuilds the probabilities and the score
-gradients of all blocks in one launch from the saved row statistics and finishes with the three
-block-sparse products of the unfused chain.
+gradients of all blocks from the saved row statistics and accumulates dq in one launch, and finishes
+with the two block-sparse products of the unfused chain that walk the columns (dk, dv).
 """
 from typing import Any, Optional, Tuple
 
@@ -33,10 +33,10 @@ class SparseAttention(torch.autograd.Function):
         rows, cols = layout.row_layout, layout.col_layout
         mm = sparse_ops.sparse_matmul
         dout = dout.contiguous()
-        # one launch for the probabilities and the score gradients, then the three products
-        p, ds = sparse_ops.sparse_attention_backward_scores(q, k, v, dout, out, lse, rows[0], rows[1],
-                                                            ctx.scale, ctx.causal, cols)
-        dq = mm(ds, k, "dsd", rows, cols, False, False) if ctx.needs_input_grad[0] else None
+        # one launch for the probabilities, the score gradients and dq, then the two products over the columns
+        p, ds, dq = sparse_ops.sparse_attention_backward_scores(q, k, v, dout, out, lse, rows[0], rows[1],
+                                                                ctx.scale, ctx.causal, cols,
+                                                                with_dq=ctx.needs_input_grad[0])
         dk = mm(ds, q, "dsd", rows, cols, True, False) if ctx.needs_input_grad[1] else None
         dv = mm(p, dout, "dsd", rows, cols, True, False) if ctx.needs_input_grad[2] else None
         return dq, dk, dv, None, None, None

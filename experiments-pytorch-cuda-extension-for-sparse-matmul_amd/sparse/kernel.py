@@ -37,7 +37,7 @@ SIGNATURES = {
     "bsa_to_sparse": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bsa_to_dense": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bsa_attention_forward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp]),
-    "bsa_attention_backward_scores": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
+    "bsa_attention_backward_scores": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
                                            _i, _i, _i, _i, _i, _f, _i, _vp]),
 }
 

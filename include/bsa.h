@@ -203,18 +203,21 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                           float scale, int causal, void *stream);
 
-/* First half of the attention backward pass in one launch: from q, k, v, the gradient `dout` of the
- * result, the forward result `out` and `lse`, the probabilities and the score gradients of every
- * stored block,
+/* The walk over the rows of the attention backward pass in one launch: from q, k, v, the gradient
+ * `dout` of the result, the forward result `out` and `lse`, the probabilities and the score
+ * gradients of every stored block, and the gradient of q,
  *   p_out  = softmax probabilities                         [batches, nnz, 32, 32]
  *   ds_out = scale * p o (dout v^T - rowsum(dout o out))   [batches, nnz, 32, 32]
- * i.e. what SDD(q, k), the softmax forward, SDD(dout, v) and the softmax backward of the unfused
- * chain produce with four launches (sparse_smm_gpu.cu:22-95 twice, sparse_softmax.cu:113-205).
- * The caller finishes with three DSD products: dq = ds k, dk = ds^T q, dv = p^T dout.
- * Same tables, schedule (any row schedule: blocks are independent here) and limits as the forward.
+ *   dq_out = ds k                                          [batches, 32 * mask_rows, head_dim]; may be NULL
+ * i.e. what SDD(q, k), the softmax forward, SDD(dout, v), the softmax backward and DSD(ds, k) of the
+ * unfused chain produce with five launches (sparse_smm_gpu.cu:22-95 twice, sparse_softmax.cu:113-205,
+ * sparse_smm_gpu.cu:106-181).  The caller finishes with the two products that walk the columns,
+ * dk = ds^T q and dv = p^T dout (bsa_matmul, mode 1, transposed first operand), and with
+ * dq = ds k as a third one if it passed dq_out = NULL.
+ * Same tables, schedule (allow_split = 0, slice_max = -1) and limits as the forward.
  */
 int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const void *v, const void *dout,
-                                  const void *out, const float *lse, void *p_out, void *ds_out,
+                                  const void *out, const float *lse, void *p_out, void *ds_out, void *dq_out,
                                   const int32_t *row_blocks, const int32_t *row_offsets,
                                   const int32_t *sched, int sched_wgs, int sched_waves,
                                   int mask_rows, int mask_cols, int nnz, int batches, int head_dim,

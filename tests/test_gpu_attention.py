@@ -122,7 +122,7 @@ def test_argument_checks():
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("name,head", [("known3x3", 64), ("rand16", 64), ("long_row_5x40", 64), ("empty_row_col_6x5", 128)])
 def test_row_statistics_and_backward_scores(name, head, causal):
-    """lse of the forward kernel, and P / dS of the one-launch backward half, against float64."""
+    """lse of the forward kernel, and P / dS / dq of the one-launch backward half, against float64."""
     from sparse.kernel import sparse_ops
     from oracle import layout_oracle as lo
     import sparse
@@ -148,8 +148,8 @@ def test_row_statistics_and_backward_scores(name, head, causal):
     got = to_np(lse)
     assert np.all(np.isposinf(got[:, ~seen]))
     assert np.max(np.abs(got[:, seen] - ref_lse[:, seen])) <= 2e-3 * max(1.0, np.max(np.abs(ref_lse[:, seen])))
-    p, ds = sparse_ops.sparse_attention_backward_scores(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), out, lse,
-                                                        rows[0], rows[1], scale, causal, cols)
+    p, ds, dq = sparse_ops.sparse_attention_backward_scores(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), out, lse,
+                                                            rows[0], rows[1], scale, causal, cols)
     pd = np.exp(s - np.where(np.isfinite(s.max(-1, keepdims=True)), s.max(-1, keepdims=True), 0))
     den = pd.sum(-1, keepdims=True)
     pd = np.divide(pd, den, out=np.zeros_like(pd), where=den > 0)
@@ -158,3 +158,7 @@ def test_row_statistics_and_backward_scores(name, head, causal):
     dsd = scale * pd * (dp - delta)
     assert rel_err(to_np(p), lo.to_sparse(mask, pd)) <= TOL
     assert rel_err(to_np(ds), lo.to_sparse(mask, dsd)) <= 2 * TOL
+    assert rel_err(to_np(dq), dsd @ to_np(k)) <= 2 * TOL          # rows without blocks: zeros
+    p2, ds2, none = sparse_ops.sparse_attention_backward_scores(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), out, lse,
+                                                                rows[0], rows[1], scale, causal, cols, with_dq=False)
+    assert none is None and torch.equal(p2, p) and torch.equal(ds2, ds)
