@@ -175,8 +175,9 @@ def main():
         attention[name + "_nnz_TFLOPs"] = round(2 * flops_one / (ms * 1e-3) / 1e12, 2)
     attention["speedup"] = round(attention["chain_us"] / attention["fused_us"], 2)
 
-    # the backward pass of the same attention: one launch for P, dS and dq + two products, against the
-    # seven launches of the unfused chain (gradients of q, k, v from dout)
+    # the backward pass of the same attention: a walk over the rows (dq) and one over the columns (dk, dv)
+    # that keep the probabilities and score gradients in registers, against the seven launches of the
+    # unfused chain (gradients of q, k, v from dout)
     from sparse.kernel import sparse_ops
     rows, cols = layout.row_layout, layout.col_layout
     for w in sets:
@@ -184,15 +185,13 @@ def main():
         w["out"], w["lse"] = sparse_ops.sparse_attention_forward(w["q"], w["k"], w["v"], rows[0], rows[1], 0.125, True,
                                                                  cols, return_lse=True)
 
-    def products(p, ds, w, with_dq=True):
-        return (sparse.matmul(ds, w["k"], "dsd", layout) if with_dq else None,
-                sparse.matmul(ds, w["q"], "dsd", layout, True, False),
+    def products(p, ds, w):
+        return (sparse.matmul(ds, w["k"], "dsd", layout), sparse.matmul(ds, w["q"], "dsd", layout, True, False),
                 sparse.matmul(p, w["dout"], "dsd", layout, True, False))
 
     def backward_fused(w):
-        p, ds, dq = sparse_ops.sparse_attention_backward_scores(w["q"], w["k"], w["v"], w["dout"], w["out"], w["lse"],
-                                                                rows[0], rows[1], 0.125, True, cols)
-        return (dq,) + products(p, ds, w, with_dq=False)[1:]
+        return sparse_ops.sparse_attention_backward(w["q"], w["k"], w["v"], w["dout"], w["out"], w["lse"],
+                                                    rows[0], rows[1], cols[0], cols[1], 0.125, True)
 
     def backward_chain(w):
         p = sparse.softmax(sparse.matmul(w["q"], w["k"], "sdd", layout, False, True), layout, 0.125, True)

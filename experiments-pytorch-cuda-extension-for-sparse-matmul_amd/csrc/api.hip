@@ -275,6 +275,28 @@ static int check_attention(const char *who, int dtype, int head_dim, const int32
     return check_schedule(sched, sched_wgs, sched_waves, batches, who);
 }
 
+static void fill_attention(bsa::AttentionArgs &p, int dtype, const void *q, const void *k, const void *v,
+                           const int32_t *blocks, const int32_t *sched, int groups, int sched_wgs, int sched_waves,
+                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim, float scale, int causal)
+{
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.blocks = blocks;
+    p.sched = sched;
+    p.groups = groups;
+    p.sched_wgs = sched_wgs;
+    p.sched_waves = sched_waves;
+    p.mask_rows = mask_rows;
+    p.mask_cols = mask_cols;
+    p.nnz = nnz;
+    p.batches = batches;
+    p.head_dim = head_dim;
+    p.scale = scale;
+    p.causal = causal != 0;
+    p.bf16 = dtype == BSA_BF16;
+}
+
 int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out, float *lse,
                           const int32_t *row_blocks, const int32_t *row_offsets,
                           const int32_t *sched, int sched_wgs, int sched_waves,
@@ -286,9 +308,11 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
                              mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
     if (!q || !k || !v || !out) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
-    bsa::AttentionArgs p{q, k, v, out, lse, nullptr, nullptr, nullptr, nullptr, nnz, row_blocks, sched, mask_rows,
-                         sched_wgs, sched_waves, mask_rows, mask_cols, batches, scale, causal != 0,
-                         dtype == BSA_BF16, head_dim};
+    bsa::AttentionArgs p;
+    fill_attention(p, dtype, q, k, v, row_blocks, sched, mask_rows, sched_wgs, sched_waves, mask_rows, mask_cols, nnz,
+                   batches, head_dim, scale, causal);
+    p.out = out;
+    p.lse = lse;
     return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
 }
 
@@ -304,12 +328,60 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
                              mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
     if (nnz == 0 && !dq_out) return BSA_OK;      // no blocks to write
-    if (!q || !k || !v || !dout || !out || !lse || (nnz > 0 && (!p_out || !ds_out)))
-        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
-    bsa::AttentionArgs p{q, k, v, const_cast<void *>(out), const_cast<float *>(lse), dout, p_out, ds_out, dq_out, nnz,
-                         row_blocks, sched, mask_rows, sched_wgs, sched_waves, mask_rows, mask_cols, batches,
-                         scale, causal != 0, dtype == BSA_BF16, head_dim};
+    if (!q || !k || !v || !dout || !out || !lse) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if ((p_out == nullptr) != (ds_out == nullptr))
+        return fail(BSA_ERR_INVALID, "%s: p_out and ds_out go together", who);
+    if (!p_out && !dq_out) return fail(BSA_ERR_INVALID, "%s: no output asked for", who);
+    bsa::AttentionArgs p;
+    fill_attention(p, dtype, q, k, v, row_blocks, sched, mask_rows, sched_wgs, sched_waves, mask_rows, mask_cols, nnz,
+                   batches, head_dim, scale, causal);
+    p.out = const_cast<void *>(out);
+    p.lse = const_cast<float *>(lse);
+    p.dout = dout;
+    p.p_out = p_out;
+    p.ds_out = ds_out;
+    p.dq_out = dq_out;
     return check_launch(bsa::launch_attention_backward_scores(p, (hipStream_t)stream), who);
+}
+
+int bsa_attention_backward(int dtype, const void *q, const void *k, const void *v, const void *dout,
+                           const void *out, const float *lse, void *dq_out, void *dk_out, void *dv_out,
+                           float *delta_ws,
+                           const int32_t *row_blocks, const int32_t *row_offsets,
+                           const int32_t *row_sched, int row_sched_wgs, int row_sched_waves,
+                           const int32_t *col_blocks, const int32_t *col_offsets,
+                           const int32_t *col_sched, int col_sched_wgs, int col_sched_waves,
+                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
+                           float scale, int causal, void *stream)
+{
+    const char *who = "bsa_attention_backward";
+    int rc = check_attention(who, dtype, head_dim, row_blocks, row_offsets, row_sched, row_sched_wgs, row_sched_waves,
+                             mask_rows, mask_cols, nnz, batches);
+    if (rc) return rc;
+    if (head_dim != 64) return fail(BSA_ERR_UNSUPPORTED, "%s: head_dim 64 is built, got %d", who, head_dim);
+    if (!col_offsets || (!col_blocks && nnz > 0)) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    rc = check_schedule(col_sched, col_sched_wgs, col_sched_waves, batches, who);
+    if (rc) return rc;
+    if (!q || !k || !v || !dout || !out || !lse || !dq_out || !dk_out || !dv_out || !delta_ws)
+        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    bsa::AttentionArgs p;
+    fill_attention(p, dtype, q, k, v, row_blocks, row_sched, mask_rows, row_sched_wgs, row_sched_waves, mask_rows,
+                   mask_cols, nnz, batches, head_dim, scale, causal);
+    p.out = const_cast<void *>(out);
+    p.lse = const_cast<float *>(lse);
+    p.dout = dout;
+    p.dq_out = dq_out;
+    p.delta = delta_ws;
+    rc = check_launch(bsa::launch_attention_backward_scores(p, (hipStream_t)stream), who);
+    if (rc) return rc;
+    p.blocks = col_blocks;
+    p.sched = col_sched;
+    p.groups = mask_cols;
+    p.sched_wgs = col_sched_wgs;
+    p.sched_waves = col_sched_waves;
+    p.dk_out = dk_out;
+    p.dv_out = dv_out;
+    return check_launch(bsa::launch_attention_backward_dkdv(p, (hipStream_t)stream), who);
 }
 
 }  // extern "C"

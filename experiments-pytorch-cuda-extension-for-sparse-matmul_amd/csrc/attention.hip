@@ -285,6 +285,7 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
     const half_t *__restrict__ dout, const half_t *__restrict__ out, const float *__restrict__ lse,
     half_t *__restrict__ p_out, half_t *__restrict__ ds_out, half_t *__restrict__ dq_out,
+    float *__restrict__ delta_out,
     const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
     int n_swg, int batches, int rows_q, int rows_k, int nnz, float scale, int causal)
 {
@@ -327,6 +328,7 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
         }
         delta += at_lane_xor32(delta);           // the other half of the head dim sits in lane l ^ 32
         const float row_lse = lse[(size_t)batch * rows_q + BS * r + qq];
+        if (delta_out != nullptr && w == e.first_wave() && h == 0) delta_out[(size_t)batch * rows_q + BS * r + qq] = delta;
 
         struct Frag { uint4 kk[KT][2], vv[KT][2]; };
         DescWindow win;
@@ -380,9 +382,11 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
                         dv[j] = narrow_16<BF>(scale * pr * (dpacc[i] - delta));
                         dsop[i >> 3][i & 7] = dv[j];
                     }
-                    const int at = 16 * kc_slot(qq, g) + 8 * h;       // 16-byte piece g of row qq, its half h
-                    *reinterpret_cast<h4 *>(lds_bytes(tile_v) + at) = pv;
-                    *reinterpret_cast<h4 *>(lds_bytes(tile_v + BS2) + at) = dv;
+                    if (p_out != nullptr) {
+                        const int at = 16 * kc_slot(qq, g) + 8 * h;   // 16-byte piece g of row qq, its half h
+                        *reinterpret_cast<h4 *>(lds_bytes(tile_v) + at) = pv;
+                        *reinterpret_cast<h4 *>(lds_bytes(tile_v + BS2) + at) = dv;
+                    }
                 }
                 if (dq_out != nullptr) {
 #pragma unroll
@@ -391,12 +395,14 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
                         for (int s = 0; s < 2; ++s)
                             dqacc[t] = mfma_16<BF>(lds_get_kc_tr_swapped(tile_k + t * BS2, s), dsop[s], dqacc[t]);
                 }
-                wave_lds_fence();
-                uint4 raw[2];
-                lds_get_linear(tile_v, raw);
-                stg_tile32(pb + (size_t)d.idx * BS2, raw);
-                lds_get_linear(tile_v + BS2, raw);
-                stg_tile32(dsb + (size_t)d.idx * BS2, raw);
+                if (p_out != nullptr) {
+                    wave_lds_fence();
+                    uint4 raw[2];
+                    lds_get_linear(tile_v, raw);
+                    stg_tile32(pb + (size_t)d.idx * BS2, raw);
+                    lds_get_linear(tile_v + BS2, raw);
+                    stg_tile32(dsb + (size_t)d.idx * BS2, raw);
+                }
             }
         }
     }
@@ -439,7 +445,7 @@ hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t 
     dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
     const size_t lds = (size_t)p.sched_waves * at_bwd_lds_per_wave(p.head_dim);
 #define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (const half_t *)p.dout, \
-                    (const half_t *)p.out, (const float *)p.lse, (half_t *)p.p_out, (half_t *)p.ds_out, (half_t *)p.dq_out, \
+                    (const half_t *)p.out, (const float *)p.lse, (half_t *)p.p_out, (half_t *)p.ds_out, (half_t *)p.dq_out, (float *)p.delta, \
                     (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
                     32 * p.mask_rows, 32 * p.mask_cols, p.nnz, p.scale, p.causal ? 1 : 0
     if (p.head_dim == 64) {
@@ -455,6 +461,187 @@ hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t 
         if (p.bf16) attention_bwd_scores_kernel<128, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
         else attention_bwd_scores_kernel<128, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
     }
+#undef BSA_AT_ARGS
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Backward, the walk over the COLUMNS: dk and dv of block column c from the blocks (r, c) of the
+// column table, with nothing but q, k, v, dO and two floats per query (lse of the forward pass,
+// delta of the row walk above) read: the probabilities and the score gradients are rebuilt in
+// registers a second time rather than stored by the row walk and read back (4 KB written + 4 KB
+// read of HBM traffic per block that this pair of kernels does not have).
+//   S  = Q_r K_c^T, dP = dO_r V_c^T    K_c and V_c stay in registers as the column operands; a lane
+//                                      holds ONE key column, 16 queries
+//   P, dS                              as in the row walk; lse and delta of the 16 queries come from a
+//                                      256-byte LDS slot
+//   dv^T += dO_r^T P,  dk^T += Q_r^T dS   the fp16 P and dS values are the column operands straight
+//                                      from the accumulators, the Q_r and dO_r tiles are read a second
+//                                      time along their rows (get_kc_tr_swapped_addr)
+// The waves of a column add their parts through LDS.  Head dim 64 only: at 128 the four accumulator
+// sets alone are 256 registers.
+// ---------------------------------------------------------------------------
+constexpr int at_bwd_col_lds_per_wave(int hd) { return 128 * hd + 256; }   // Q tiles + dO tiles (= one parked accumulator set) + stats
+
+template <int HD, bool BF>
+__global__ __launch_bounds__(512) void attention_bwd_dkdv_kernel(
+    const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
+    const half_t *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ delta,
+    half_t *__restrict__ dk_out, half_t *__restrict__ dv_out,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int rows_q, int rows_k, float scale, int causal)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const bool active = e.group >= 0;
+    const int c = e.group;
+    const int key = l & 31, h = l >> 5;          // key column of this lane, lane half
+    constexpr int KT = HD / 32, LDS_PER_WAVE = at_bwd_col_lds_per_wave(HD);
+    const float scale2 = scale * 1.4426950408889634f;
+
+    unsigned char *my_lds = lds_raw + (size_t)w * LDS_PER_WAVE;
+    half_t *tile_q = reinterpret_cast<half_t *>(my_lds);
+    half_t *tile_do = tile_q + KT * BS2;
+    float *stats = reinterpret_cast<float *>(my_lds + 128 * HD);      // 32 lse, 32 delta of the block's queries
+    const half_t *qb = q + (size_t)batch * rows_q * HD;
+    const half_t *dob = dout + (size_t)batch * rows_q * HD;
+    const float *lse_b = lse + (size_t)batch * rows_q;
+    const float *delta_b = delta + (size_t)batch * rows_q;
+
+    f16v dvacc[KT], dkacc[KT];                   // dv^T, dk^T: lane = key column, values = head dims as in the forward kernel
+#pragma unroll
+    for (int t = 0; t < KT; ++t) dvacc[t] = dkacc[t] = f16v{0};
+
+    if (active && e.begin < e.end) {
+        // column operands of the first two products: lane (key, h) holds d = 16 s + 8 h .. + 7 of its key
+        const size_t koff = ((size_t)batch * rows_k + BS * c + key) * HD + 8 * h;
+        h8 kop[HD / 16], vop[HD / 16];
+#pragma unroll
+        for (int s = 0; s < HD / 16; ++s) {
+            kop[s] = as_h8(ldg16(k + koff + 16 * s));
+            vop[s] = as_h8(ldg16(v + koff + 16 * s));
+        }
+        struct Frag { uint4 qq[KT][2], dd[KT][2]; float stat; };
+        DescWindow win;
+        auto load = [&](int p, Frag &f) {
+            const int r = win.get(p).row();
+#pragma unroll
+            for (int dt = 0; dt < KT; ++dt) {
+                ldg_tile32(qb + (size_t)(BS * r) * HD + 32 * dt, HD, f.qq[dt]);
+                ldg_tile32(dob + (size_t)(BS * r) * HD + 32 * dt, HD, f.dd[dt]);
+            }
+            f.stat = h == 0 ? lse_b[BS * r + key] : delta_b[BS * r + key];
+        };
+        Frag fr;
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+            load(seg, fr);
+            for (int p = seg; p < seg_end; ++p) {
+                const int r = win.get(p).row();
+                wave_lds_fence();
+#pragma unroll
+                for (int dt = 0; dt < KT; ++dt) {
+                    lds_put_kc<false>(tile_q + dt * BS2, fr.qq[dt]);
+                    lds_put_kc<false>(tile_do + dt * BS2, fr.dd[dt]);
+                }
+                stats[l] = fr.stat;
+                wave_lds_fence();
+                if (p + 1 < seg_end) load(p + 1, fr);
+                f16v sacc = {0}, dpacc = {0};
+#pragma unroll
+                for (int dt = 0; dt < KT; ++dt)
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        sacc = mfma_16<BF>(lds_get_kc(tile_q + dt * BS2, s), kop[2 * dt + s], sacc);
+                        dpacc = mfma_16<BF>(lds_get_kc(tile_do + dt * BS2, s), vop[2 * dt + s], dpacc);
+                    }
+                // accumulator value i of lane half h is query 8 (i / 4) + 4 h + i % 4 of this lane's key
+                h8 pop[2], dsop[2];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float4 ls = *reinterpret_cast<const float4 *>(stats + 8 * g + 4 * h);
+                    const float4 dl = *reinterpret_cast<const float4 *>(stats + 32 + 8 * g + 4 * h);
+                    const float lsv[4] = {ls.x, ls.y, ls.z, ls.w}, dlv[4] = {dl.x, dl.y, dl.z, dl.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int i = 4 * g + j, qrow = 8 * g + 4 * h + j;
+                        float pr = at_exp2(__builtin_fmaf(sacc[i], scale2, -lsv[j]));
+                        if (causal && (c > r || (c == r && key > qrow))) pr = 0.f;
+                        pop[i >> 3][i & 7] = narrow_16<BF>(pr);
+                        dsop[i >> 3][i & 7] = narrow_16<BF>(scale * pr * (dpacc[i] - dlv[j]));
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < KT; ++t)
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        dvacc[t] = mfma_16<BF>(lds_get_kc_tr_swapped(tile_do + t * BS2, s), pop[s], dvacc[t]);
+                        dkacc[t] = mfma_16<BF>(lds_get_kc_tr_swapped(tile_q + t * BS2, s), dsop[s], dkacc[t]);
+                    }
+            }
+        }
+    }
+
+    // team merge, one accumulator set at a time (the staging tiles hold exactly one): every wave of a
+    // column but the leader parks its part, the leader adds and stores
+    const int slot0 = e.first_wave(), nw = e.team_waves();
+    const bool leader = active && w == slot0;
+    float *park = reinterpret_cast<float *>(my_lds);
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        f16v (&acc)[KT] = which == 0 ? dvacc : dkacc;
+        if (which == 1) __syncthreads();         // the leaders have read the first set
+        if (active && !leader) {
+            wave_lds_fence();
+#pragma unroll
+            for (int t = 0; t < KT; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) park[(t * 16 + i) * WAVE + l] = acc[t][i];
+        }
+        __syncthreads();
+        if (leader) {
+            for (int o = 1; o < nw; ++o) {
+                const float *op = reinterpret_cast<const float *>(lds_raw + (size_t)(w + o) * LDS_PER_WAVE);
+#pragma unroll
+                for (int t = 0; t < KT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[t][i] += op[(t * 16 + i) * WAVE + l];
+            }
+            half_t *drow = (which == 0 ? dv_out : dk_out) + ((size_t)batch * rows_k + BS * c + key) * HD + 4 * h;
+#pragma unroll
+            for (int t = 0; t < KT; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    h4 o;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) o[j] = narrow_16<BF>(acc[t][4 * g + j]);
+                    *reinterpret_cast<h4 *>(drow + 32 * t + 8 * g) = o;
+                }
+        }
+    }
+}
+
+hipError_t launch_attention_backward_dkdv(const AttentionArgs &p, hipStream_t st)
+{
+    dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
+    const size_t lds = (size_t)p.sched_waves * at_bwd_col_lds_per_wave(64);
+#define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (const half_t *)p.dout, \
+                    (const float *)p.lse, (const float *)p.delta, (half_t *)p.dk_out, (half_t *)p.dv_out, \
+                    (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
+                    32 * p.mask_rows, 32 * p.mask_cols, p.scale, p.causal ? 1 : 0
+    if (lds > 65536) {
+        const void *fn = p.bf16 ? (const void *)attention_bwd_dkdv_kernel<64, true>
+                                : (const void *)attention_bwd_dkdv_kernel<64, false>;
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    if (p.bf16) attention_bwd_dkdv_kernel<64, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
+    else attention_bwd_dkdv_kernel<64, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
 #undef BSA_AT_ARGS
     return hipGetLastError();
 }

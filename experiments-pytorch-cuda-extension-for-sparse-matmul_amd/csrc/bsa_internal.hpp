@@ -57,25 +57,29 @@ hipError_t launch_softmax_forward(int dtype, const SoftmaxArgs &p, hipStream_t s
 hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t stream);
 
 struct AttentionArgs {
-    const void *q, *k, *v;
-    void *out;              // forward: result; backward: the forward result (read)
-    void *lse;              // forward: optional output; backward: input
-    const void *dout;       // backward only
-    void *p_out, *ds_out;   // backward only: [batches, nnz, 32, 32] each
-    void *dq_out;           // backward only, may be null: [batches, 32 mask_rows, head_dim]
-    int nnz;
-    const int32_t *blocks;
-    const int32_t *sched;
-    int groups;
-    int sched_wgs, sched_waves;
-    int mask_rows, mask_cols, batches;
-    float scale;
-    bool causal;
-    bool bf16;      // operands are bfloat16, not fp16
-    int head_dim;   // 64 or 128
+    const void *q = nullptr, *k = nullptr, *v = nullptr;
+    void *out = nullptr;            // forward: result; backward: the forward result (read)
+    void *lse = nullptr;            // forward: optional output; backward: input
+    const void *dout = nullptr;     // backward only
+    void *p_out = nullptr, *ds_out = nullptr;   // row walk of the backward pass, both or neither: [batches, nnz, 32, 32]
+    void *dq_out = nullptr;         // row walk, may be null: [batches, 32 mask_rows, head_dim]
+    void *delta = nullptr;          // float [batches, 32 mask_rows], rowsum(dout o out): written by the row walk (may be
+                                    // null there), read by the column walk
+    void *dk_out = nullptr, *dv_out = nullptr;  // column walk: [batches, 32 mask_cols, head_dim]
+    int nnz = 0;
+    const int32_t *blocks = nullptr;
+    const int32_t *sched = nullptr;
+    int groups = 0;                 // block rows (block columns for the column walk)
+    int sched_wgs = 0, sched_waves = 0;
+    int mask_rows = 0, mask_cols = 0, batches = 0;
+    float scale = 1.f;
+    bool causal = false;
+    bool bf16 = false;      // operands are bfloat16, not fp16
+    int head_dim = 64;      // 64 or 128
 };
 
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t stream);
 hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t stream);
+hipError_t launch_attention_backward_dkdv(const AttentionArgs &p, hipStream_t stream);   // groups = block columns, head dim 64
 
 }  // namespace bsa

@@ -18,6 +18,7 @@ SCHEDULE_SDD = (4, 2)
 SCHEDULE_SOFTMAX = (4, 4)
 SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
 SCHEDULE_ATTENTION_BACKWARD = (16, 4)
+SCHEDULE_ATTENTION_BACKWARD_COLUMNS = (8, 8)
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
@@ -309,3 +310,35 @@ def sparse_attention_backward_scores(q, k, v, dout, out, lse, row_blocks, row_ta
                 sched.table.data_ptr(), sched.workgroups, sched.waves, mask_rows, mask_cols, nnz, batches, head,
                 float(scale), int(bool(causal)), _k.current_stream()))
     return p, ds, dq
+
+
+def sparse_attention_backward(q, k, v, dout, out, lse, row_blocks, row_table, col_blocks, col_table, scale=1.0,
+                              causal=False):
+    """``(dq, dk, dv)`` of the fused attention in two launches (a walk over the rows, one over the
+    columns), the probabilities and score gradients rebuilt in registers in both instead of stored:
+    the seven launches of the unfused backward chain (sparse/matmul.py:27-52, sparse_softmax.cu:165-205)
+    without a block stack in memory.  fp16 / bf16, head dim 64."""
+    col_layout = (col_blocks, col_table)
+    _check_layout(col_layout, "col_layout")
+    row_layout, mask_rows, mask_cols, nnz, head, batches = _attention_common(q, k, v, row_blocks, row_table,
+                                                                              col_layout)
+    if head != 64:
+        raise ValueError(f"the two-launch backward is built for head dim 64, got {head}")
+    if dout.shape != q.shape or out.shape != q.shape or dout.dtype != q.dtype or out.dtype != q.dtype:
+        raise ValueError("dout and out must match q in shape and dtype")
+    if lse.dtype != torch.float32 or lse.shape != q.shape[:-1]:
+        raise ValueError("lse must be the float32 row statistics of the forward pass")
+    q, k, v, dout, out, lse = (t.contiguous() for t in (q, k, v, dout, out, lse))
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if q.numel() > 0:
+        delta = torch.empty_like(lse)
+        rs = schedule_for(row_layout, SCHEDULE_ATTENTION_BACKWARD + (False,))
+        cs = schedule_for(col_layout, SCHEDULE_ATTENTION_BACKWARD_COLUMNS + (False,))
+        with torch.cuda.device(q.device):
+            _k.check(_k.lib.bsa_attention_backward(
+                _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
+                lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(),
+                row_blocks.data_ptr(), row_table.data_ptr(), rs.table.data_ptr(), rs.workgroups, rs.waves,
+                col_blocks.data_ptr(), col_table.data_ptr(), cs.table.data_ptr(), cs.workgroups, cs.waves,
+                mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), _k.current_stream()))
+    return dq, dk, dv

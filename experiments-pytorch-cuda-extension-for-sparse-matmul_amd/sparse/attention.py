@@ -2,9 +2,10 @@
 
 The reference has no such call: its users chain ``matmul(q, k, 'sdd', layout, False, True)``, a
 softmax and ``matmul(p, v, 'dsd', layout)`` (``sparse/matmul.py:57``).  The forward here is ONE
-launch that keeps the scores on the chip; the backward rebuilds the probabilities and the score
-gradients of all blocks from the saved row statistics and accumulates dq in one launch, and finishes
-with the two block-sparse products of the unfused chain that walk the columns (dk, dv).
+launch that keeps the scores on the chip.  The backward at head dim 64 is two launches that rebuild
+the probabilities and the score gradients in registers from the saved row statistics, one walking
+the rows (dq), one the columns (dk, dv); at head dim 128 one launch stores them and accumulates dq,
+and the two block-sparse products of the unfused chain that walk the columns finish (dk, dv).
 """
 from typing import Any, Optional, Tuple
 
@@ -33,7 +34,13 @@ class SparseAttention(torch.autograd.Function):
         rows, cols = layout.row_layout, layout.col_layout
         mm = sparse_ops.sparse_matmul
         dout = dout.contiguous()
-        # one launch for the probabilities, the score gradients and dq, then the two products over the columns
+        if q.size(-1) == 64:
+            # two launches, nothing stored per block: a walk over the rows for dq, one over the columns for dk and dv
+            dq, dk, dv = sparse_ops.sparse_attention_backward(q, k, v, dout, out, lse, rows[0], rows[1], cols[0],
+                                                              cols[1], ctx.scale, ctx.causal)
+            return dq, dk, dv, None, None, None
+        # head dim 128: one launch for the probabilities, the score gradients and dq, then the two products
+        # over the columns
         p, ds, dq = sparse_ops.sparse_attention_backward_scores(q, k, v, dout, out, lse, rows[0], rows[1],
                                                                 ctx.scale, ctx.causal, cols,
                                                                 with_dq=ctx.needs_input_grad[0])

@@ -39,6 +39,8 @@ SIGNATURES = {
     "bsa_attention_forward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "bsa_attention_backward_scores": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
                                            _i, _i, _i, _i, _i, _f, _i, _vp]),
+    "bsa_attention_backward": (_i, [_i] + [_vp] * 10 + [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i,
+                                                        _i, _i, _i, _i, _i, _f, _i, _vp]),
 }
 
 

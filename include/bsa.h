@@ -223,6 +223,27 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
                                   int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                                   float scale, int causal, void *stream);
 
+/* The whole backward pass of that operator in two launches, with no block stack in memory: a walk over
+ * the rows that rebuilds the probabilities and the score gradients in registers and accumulates
+ *   dq_out = ds k                       [batches, 32 * mask_rows, head_dim]
+ * (and leaves rowsum(dout o out) in `delta_ws`, float [batches, 32 * mask_rows], caller-provided), and
+ * a walk over the columns that rebuilds them a second time and accumulates
+ *   dk_out = ds^T q,  dv_out = p^T dout [batches, 32 * mask_cols, head_dim].
+ * Seven launches in the unfused chain (sparse/matmul.py:27-52 three times over, sparse_softmax_op.cu:43-63).
+ * Row tables and schedule as for bsa_attention_forward; column tables with a schedule of their own built the
+ * same way (allow_split = 0, slice_max = -1) on col_offsets.  fp16 / bf16, head_dim 64 only
+ * (BSA_ERR_UNSUPPORTED otherwise: use bsa_attention_backward_scores and two bsa_matmul calls).
+ */
+int bsa_attention_backward(int dtype, const void *q, const void *k, const void *v, const void *dout,
+                           const void *out, const float *lse, void *dq_out, void *dk_out, void *dv_out,
+                           float *delta_ws,
+                           const int32_t *row_blocks, const int32_t *row_offsets,
+                           const int32_t *row_sched, int row_sched_wgs, int row_sched_waves,
+                           const int32_t *col_blocks, const int32_t *col_offsets,
+                           const int32_t *col_sched, int col_sched_wgs, int col_sched_waves,
+                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
+                           float scale, int causal, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -100,3 +100,27 @@ def test_other_entry_points_validate(k):
     assert k.lib.bsa_matmul_workspace_bytes(0, 4, 2, 3, 128, 128) == 0
     assert k.lib.bsa_matmul_workspace_bytes(1, 0, 0, 3, 128, 128) == 0
     assert k.lib.bsa_matmul_workspace_bytes(1, 4, 2, 3, 128, 128) == 256 + 4 * 3 * 2 * 8192
+
+
+def test_attention_entry_points_validate(k):
+    """Argument checks of the fused attention calls; every case returns before a launch."""
+    fwd = lambda dtype=1, head=64, q=P, rows=4, cols=4, nnz=5, batches=1, wgs=4, waves=4: k.lib.bsa_attention_forward(
+        dtype, q, P, P, P, None, P, P, P, wgs, waves, rows, cols, nnz, batches, head, 1.0, 0, None)
+    assert fwd(dtype=0) == -3 and "fp16" in k.lib.bsa_last_error().decode()
+    assert fwd(head=32) == -3 and "head_dim" in k.lib.bsa_last_error().decode()
+    assert fwd(q=None) == -1
+    assert fwd(nnz=17) == -1 and "nnz" in k.lib.bsa_last_error().decode()
+    assert fwd(rows=0) == -1 and fwd(batches=0) == -1 and fwd(waves=9) == -1
+
+    scores = lambda p=P, ds=P, dq=P, head=64, lse=P: k.lib.bsa_attention_backward_scores(
+        1, P, P, P, P, P, lse, p, ds, dq, P, P, P, 4, 4, 4, 4, 5, 1, head, 1.0, 0, None)
+    assert scores(ds=None) == -1 and "go together" in k.lib.bsa_last_error().decode()
+    assert scores(p=None, ds=None, dq=None) == -1 and "no output" in k.lib.bsa_last_error().decode()
+    assert scores(lse=None) == -1
+    assert scores(head=96) == -3
+
+    full = lambda head=64, dk=P, delta=P, col_sched=P, col_waves=4: k.lib.bsa_attention_backward(
+        1, P, P, P, P, P, P, P, dk, P, delta, P, P, P, 4, 4, P, P, col_sched, 4, col_waves, 4, 4, 5, 1, head, 1.0, 0, None)
+    assert full(head=128) == -3 and "head_dim 64" in k.lib.bsa_last_error().decode()
+    assert full(dk=None) == -1 and full(delta=None) == -1
+    assert full(col_sched=None) == -1 and full(col_waves=0) == -1

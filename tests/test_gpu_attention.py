@@ -162,3 +162,43 @@ def test_row_statistics_and_backward_scores(name, head, causal):
     p2, ds2, none = sparse_ops.sparse_attention_backward_scores(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), out, lse,
                                                                 rows[0], rows[1], scale, causal, cols, with_dq=False)
     assert none is None and torch.equal(p2, p) and torch.equal(ds2, ds)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name", ["known3x3", "rand16", "long_row_5x40", "empty_row_col_6x5", "long_col_70x3", "full4",
+                                  "tall_7x2", "wide_2x9", "one_cell"])
+def test_two_launch_backward(name, dtype, causal):
+    """dq, dk, dv of the row walk + column walk (nothing stored per block) against float64."""
+    from sparse.kernel import sparse_ops
+    import sparse
+    mask = np.asarray(ZOO[name])
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    q, k, v = (t.to(dtype) for t in _qkv(mask, seed=23, head=64))
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(24)).to(dtype)
+    scale = 0.13
+    rows, cols = L.row_layout, L.col_layout
+    out, lse = sparse_ops.sparse_attention_forward(q.cuda(), k.cuda(), v.cuda(), rows[0], rows[1], scale, causal,
+                                                   cols, return_lse=True)
+    dq, dk, dv = sparse_ops.sparse_attention_backward(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), out, lse,
+                                                      rows[0], rows[1], cols[0], cols[1], scale, causal)
+    vis = np.repeat(np.repeat(mask != 0, 32, 0), 32, 1)
+    if causal:
+        r_, c_ = np.indices(vis.shape)
+        vis &= c_ <= r_
+    qn, kn, vn, dn = (to_np(t.float()) for t in (q, k, v, dout))
+    s = np.where(vis, scale * np.einsum("bqd,bkd->bqk", qn, kn), -np.inf)
+    top = s.max(-1, keepdims=True)
+    pd = np.exp(s - np.where(np.isfinite(top), top, 0))
+    den = pd.sum(-1, keepdims=True)
+    pd = np.divide(pd, den, out=np.zeros_like(pd), where=den > 0)
+    dp = np.einsum("bqd,bkd->bqk", dn, vn)
+    # delta from the rounded forward result, as the kernels take it
+    delta = np.sum(dn * to_np(out.float()), -1, keepdims=True)
+    dsd = scale * pd * (dp - delta)
+    tol = 4 * TOL if dtype == torch.float16 else 2e-2
+    assert rel_err(to_np(dq.float()), dsd @ kn) <= tol
+    assert rel_err(to_np(dk.float()), np.einsum("bqk,bqd->bkd", dsd, qn)) <= tol
+    assert rel_err(to_np(dv.float()), np.einsum("bqk,bqd->bkd", pd, dn)) <= tol
+    # columns and rows without blocks get zeros, not stale memory
+    assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all()
