@@ -16,7 +16,7 @@ launch finds its operands in HBM, not in the 256 MB infinity cache (`--sets 1`
 shows the cache-resident figures).  Launches are replayed
 from HIP graphs (the Python call path costs more than a 10 us kernel).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sets S] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sets S] [--no-cpu] [--no-attention]
 """
 import argparse
 import json
@@ -40,6 +40,8 @@ def main():
                     help="operand sets to rotate over (1 = the same operands every launch, which the 256 MB "
                          "infinity cache then serves)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-attention", action="store_true",
+                    help="skip the fused attention legs (kernel traces of the hot path alone)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -155,57 +157,59 @@ def main():
             per_op[name]["nnz_TFLOPs"] = round(tf, 2)
             per_op[name]["mfma_frac"] = round(tf / MFMA_F16_PEAK_TFLOPS, 4)
 
-    # attention forward as a whole, q k v -> out: one fused launch against the chain of three launches
-    # (the two products of a forward pass are 2 * flops_one); not part of `value`
-    def chain(w):
-        s = sparse.matmul(w["q"], w["k"], "sdd", layout, False, True)
-        return sparse.matmul(sparse.softmax(s, layout, 0.125, True), w["v"], "dsd", layout)
+    attention = None
+    if not args.no_attention:
+        # attention forward as a whole, q k v -> out: one fused launch against the chain of three launches
+        # (the two products of a forward pass are 2 * flops_one); not part of `value`
+        def chain(w):
+            s = sparse.matmul(w["q"], w["k"], "sdd", layout, False, True)
+            return sparse.matmul(sparse.softmax(s, layout, 0.125, True), w["v"], "dsd", layout)
 
-    def fused(w):
-        return sparse.attention(w["q"], w["k"], w["v"], layout, 0.125, True)
+        def fused(w):
+            return sparse.attention(w["q"], w["k"], w["v"], layout, 0.125, True)
 
-    with torch.no_grad():
-        a, b = fused(sets[0]), chain(sets[0])
-        err = ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
-        assert err <= 2e-3, f"fused attention differs from the chain: {err}"
-    attention = {}
-    for name, fn in (("fused", fused), ("chain", chain)):
-        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
-        attention[name + "_us"] = round(ms * 1e3, 3)
-        attention[name + "_nnz_TFLOPs"] = round(2 * flops_one / (ms * 1e-3) / 1e12, 2)
-    attention["speedup"] = round(attention["chain_us"] / attention["fused_us"], 2)
-
-    # the backward pass of the same attention: a walk over the rows (dq) and one over the columns (dk, dv)
-    # that keep the probabilities and score gradients in registers, against the seven launches of the
-    # unfused chain (gradients of q, k, v from dout)
-    from sparse.kernel import sparse_ops
-    rows, cols = layout.row_layout, layout.col_layout
-    for w in sets:
-        w["dout"] = torch.randn_like(w["q"])
-        w["out"], w["lse"] = sparse_ops.sparse_attention_forward(w["q"], w["k"], w["v"], rows[0], rows[1], 0.125, True,
-                                                                 cols, return_lse=True)
-
-    def products(p, ds, w):
-        return (sparse.matmul(ds, w["k"], "dsd", layout), sparse.matmul(ds, w["q"], "dsd", layout, True, False),
-                sparse.matmul(p, w["dout"], "dsd", layout, True, False))
-
-    def backward_fused(w):
-        return sparse_ops.sparse_attention_backward(w["q"], w["k"], w["v"], w["dout"], w["out"], w["lse"],
-                                                    rows[0], rows[1], cols[0], cols[1], 0.125, True)
-
-    def backward_chain(w):
-        p = sparse.softmax(sparse.matmul(w["q"], w["k"], "sdd", layout, False, True), layout, 0.125, True)
-        dp = sparse.matmul(w["dout"], w["v"], "sdd", layout, False, True)
-        ds = sparse_ops.sparse_softmax_backward(p, dp, rows[0], rows[1], 0.125, cols)
-        return products(p, ds, w)
-
-    with torch.no_grad():
-        for a, b in zip(backward_fused(sets[0]), backward_chain(sets[0])):
+        with torch.no_grad():
+            a, b = fused(sets[0]), chain(sets[0])
             err = ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
-            assert err <= 4e-3, f"attention backward differs from the chain: {err}"
-    for name, fn in (("backward_us", backward_fused), ("backward_chain_us", backward_chain)):
-        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
-        attention[name] = round(ms * 1e3, 3)
+            assert err <= 2e-3, f"fused attention differs from the chain: {err}"
+        attention = {}
+        for name, fn in (("fused", fused), ("chain", chain)):
+            ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+            attention[name + "_us"] = round(ms * 1e3, 3)
+            attention[name + "_nnz_TFLOPs"] = round(2 * flops_one / (ms * 1e-3) / 1e12, 2)
+        attention["speedup"] = round(attention["chain_us"] / attention["fused_us"], 2)
+
+        # the backward pass of the same attention: a walk over the rows (dq) and one over the columns (dk, dv)
+        # that keep the probabilities and score gradients in registers, against the seven launches of the
+        # unfused chain (gradients of q, k, v from dout)
+        from sparse.kernel import sparse_ops
+        rows, cols = layout.row_layout, layout.col_layout
+        for w in sets:
+            w["dout"] = torch.randn_like(w["q"])
+            w["out"], w["lse"] = sparse_ops.sparse_attention_forward(w["q"], w["k"], w["v"], rows[0], rows[1], 0.125, True,
+                                                                     cols, return_lse=True)
+
+        def products(p, ds, w):
+            return (sparse.matmul(ds, w["k"], "dsd", layout), sparse.matmul(ds, w["q"], "dsd", layout, True, False),
+                    sparse.matmul(p, w["dout"], "dsd", layout, True, False))
+
+        def backward_fused(w):
+            return sparse_ops.sparse_attention_backward(w["q"], w["k"], w["v"], w["dout"], w["out"], w["lse"],
+                                                        rows[0], rows[1], cols[0], cols[1], 0.125, True)
+
+        def backward_chain(w):
+            p = sparse.softmax(sparse.matmul(w["q"], w["k"], "sdd", layout, False, True), layout, 0.125, True)
+            dp = sparse.matmul(w["dout"], w["v"], "sdd", layout, False, True)
+            ds = sparse_ops.sparse_softmax_backward(p, dp, rows[0], rows[1], 0.125, cols)
+            return products(p, ds, w)
+
+        with torch.no_grad():
+            for a, b in zip(backward_fused(sets[0]), backward_chain(sets[0])):
+                err = ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+                assert err <= 4e-3, f"attention backward differs from the chain: {err}"
+        for name, fn in (("backward_us", backward_fused), ("backward_chain_us", backward_chain)):
+            ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+            attention[name] = round(ms * 1e3, 3)
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/): same
     # workload, same kernels; absent file -> null
