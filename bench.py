@@ -16,7 +16,7 @@ launch finds its operands in HBM, not in the 256 MB infinity cache (`--sets 1`
 shows the cache-resident figures).  Launches are replayed
 from HIP graphs (the Python call path costs more than a 10 us kernel).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sets S] [--no-cpu] [--no-attention]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sets S] [--no-cpu] [--no-attention] [--no-dense] [--no-configs]
 """
 import argparse
 import json
@@ -42,6 +42,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-attention", action="store_true",
                     help="skip the fused attention legs (kernel traces of the hot path alone)")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense torch.matmul yardstick")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -211,6 +213,111 @@ def main():
             ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
             attention[name] = round(ms * 1e3, 3)
 
+    def graph_time_us(fn, reps, iters=10):
+        """Average duration of one call of fn(), `reps` calls per HIP graph, on its own operands."""
+        with torch.cuda.stream(stream), torch.no_grad():
+            fn()
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                keep = [fn() for _ in range(reps)]
+            for _ in range(2):
+                g.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for _ in range(iters):
+                g.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            del keep
+        return e0.elapsed_time(e1) / (iters * reps) * 1e3
+
+    # The same three products as DENSE fp16 matmuls at the full M, N, K (torch.matmul: rocBLAS / hipBLASLt),
+    # the "dense-MFMA-equivalent" yardstick: what the library reaches when it multiplies all 16384 blocks
+    # of a head, against what these kernels reach on the 1530 stored ones.
+    dense_equivalent = None
+    if not args.no_dense:
+        w = sets[0]
+        with torch.no_grad():
+            p_dense = layout.to_dense(w["scores"])                  # [16, 4096, 4096]
+            w_dense = layout.to_dense(w["w"])
+            kt, dyt = w["k"].transpose(-1, -2), w["v"].transpose(-1, -2)
+        dense_flops = 2.0 * seq * seq * D * B
+        dense_equivalent = {}
+        for name, fn in (("sdd", lambda: torch.matmul(w["q"], kt)), ("dsd", lambda: torch.matmul(p_dense, w["v"])),
+                         ("dds", lambda: torch.matmul(dyt, w_dense))):
+            us = graph_time_us(fn, 4)
+            dtf = dense_flops / (us * 1e-6) / 1e12
+            dense_equivalent[name] = {
+                "dense_us": round(us, 2), "dense_TFLOPs": round(dtf, 1),
+                "dense_mfma_frac": round(dtf / MFMA_F16_PEAK_TFLOPS, 4),
+                "nnz_TFLOPs_over_dense_TFLOPs": round(per_op[name]["nnz_TFLOPs"] / dtf, 3),
+                "time_dense_over_sparse": round(us / per_op[name]["us"], 2)}
+        del p_dense, w_dense
+
+    # the five configurations of the coverage table, each on its own operands (one set: the small ones are
+    # cache-resident), per launch from a HIP graph and eagerly (Python call path included)
+    configs = None
+    if not args.no_configs:
+        import time
+        configs = {}
+
+        def run_config(name, fn, reps, flops=None, nbytes=None):
+            us = graph_time_us(fn, reps)
+            with torch.no_grad():
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(50):
+                    fn()
+                torch.cuda.synchronize()
+                eager = (time.perf_counter() - t0) / 50 * 1e6
+            row = {"us": round(us, 2), "eager_us": round(eager, 1)}
+            if flops:
+                row["nnz_TFLOPs"] = round(flops / (us * 1e-6) / 1e12, 2)
+            if nbytes:
+                row["GBps"] = round(nbytes / (us * 1e-6) / 1e9, 1)
+                row["hbm_frac"] = round(row["GBps"] / HBM_PEAK_GBS, 4)
+            configs[name] = row
+
+        def on_gpu(c):
+            return {k: (v.to(dev) if hasattr(v, "to") else v) for k, v in c.items()}
+
+        c = on_gpu(wl.config1())
+        l1 = sparse.SparseLayout(c["mask"])
+        run_config("config1_sdd_fp32_16x16", lambda: sparse.matmul(c["a"], c["b"], "sdd", l1, False, True), 20,
+                   flops=2.0 * l1.num_blocks * 32 * 32 * 64,
+                   nbytes=(2 * 512 * 64 + l1.num_blocks * 1024) * 4)
+        c2 = on_gpu(wl.config2())
+        l2 = sparse.SparseLayout(c2["mask"])
+        run_config("config2_dsd_fp16_64x64_local", lambda: sparse.matmul(c2["a"], c2["b"], "dsd", l2), 20,
+                   flops=2.0 * l2.num_blocks * 32 * 32 * 64 * 16,
+                   nbytes=(l2.num_blocks * 1024 + 2 * 2048 * 64) * 16 * 2)
+        c3 = on_gpu(wl.config3())
+        run_config("config3_softmax_fp16_causal", lambda: sparse.softmax(c3["x"], layout, 0.125, True), 12,
+                   nbytes=2 * nnz * 1024 * 16 * 2)
+        c4 = on_gpu(wl.config4())
+        run_config("config4_dds_fp16", lambda: sparse.matmul(c4["a"], c4["b"], "dds", layout, True, False), 12,
+                   flops=flops_one, nbytes=bytes_alg["dds"])
+        run_config("config4_as_dsd_TF", lambda: sparse.matmul(c4["b"], c4["a"], "dsd", layout, True, False), 12,
+                   flops=flops_one, nbytes=bytes_alg["dds"])
+        del c, c2, c3, c4
+        c5 = on_gpu(wl.config5())
+        l5 = sparse.SparseLayout(c5["mask"])
+        n5, b5 = l5.num_blocks, 48
+
+        def chain5():
+            sc = sparse.matmul(c5["q"], c5["k"], "sdd", l5, False, True)
+            return sparse.matmul(sparse.softmax(sc, l5, 0.125, False), c5["v"], "dsd", l5)
+
+        f5 = 2 * 2.0 * n5 * 32 * 32 * 64 * b5
+        run_config("config5_chain_sdd_softmax_dsd_fp16_8192", chain5, 4, flops=f5,
+                   nbytes=(4 * 8192 * 64 + 4 * n5 * 1024) * b5 * 2)
+        run_config("config5_fused_attention", lambda: sparse.attention(c5["q"], c5["k"], c5["v"], l5, 0.125, False), 4,
+                   flops=f5, nbytes=4 * 8192 * 64 * b5 * 2)
+        configs["config5_nnz"] = n5
+        del c5
+
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/): same
     # workload, same kernels; absent file -> null
     traffic = {}
@@ -240,6 +347,8 @@ def main():
                                  "traffic": traffic.get("softmax")}},
         "kernels": per_op,
         "attention": attention,
+        "dense_equivalent": dense_equivalent,
+        "configs": configs,
     }
 
     if not args.no_cpu:

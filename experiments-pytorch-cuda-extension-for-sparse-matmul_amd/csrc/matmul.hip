@@ -251,14 +251,24 @@ __global__ __launch_bounds__(512) void sdd_f32_kernel(
         const BlockDesc d = win.get(p);
         const int cblk = d.col();
         f16v acc = {0};
-        for (int kb = 0; kb < kbs; ++kb) {
-            float av[16], bv[16];
+        auto load = [&](int kb, float (&av)[16], float (&bv)[16]) {
             if (A_KC) ldg_tile_f32<true, false>(ab + (size_t)(BS * r) * K + BS * kb, K, av);
             else ldg_tile_f32<false, false>(ab + (size_t)(BS * kb) * M + BS * r, M, av);
             if (B_KC) ldg_tile_f32<true, true>(bb + (size_t)(BS * cblk) * K + BS * kb, K, bv);
             else ldg_tile_f32<false, true>(bb + (size_t)(BS * kb) * N + BS * cblk, N, bv);
+        };
+        // two k-blocks per round: both sets of loads are in flight before the first product
+        for (int kb = 0; kb < kbs; kb += 2) {
+            float av0[16], bv0[16], av1[16], bv1[16];
+            const bool two = kb + 1 < kbs;
+            load(kb, av0, bv0);
+            if (two) load(kb + 1, av1, bv1);
 #pragma unroll
-            for (int t = 0; t < 16; ++t) acc = mfma_f32(bv[t], av[t], acc);
+            for (int t = 0; t < 16; ++t) acc = mfma_f32(bv0[t], av0[t], acc);
+            if (two) {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) acc = mfma_f32(bv1[t], av1[t], acc);
+            }
         }
         store16_f32(cb + (size_t)d.idx * BS2 + (l & 31) * BS + 16 * (l >> 5), acc);
     }

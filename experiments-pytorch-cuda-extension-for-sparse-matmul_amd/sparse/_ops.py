@@ -15,6 +15,7 @@ SCHEDULE_GROUP_WALK = (12, 2)        # groups of at most GROUP_WALK_LONG pairs (
 SCHEDULE_GROUP_WALK_LONG = (8, 4)    # tables with longer groups (columns of causal / strided masks)
 GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
+SCHEDULE_SDD_F32 = (1, 4)              # fp32 SDD reloads both operands per block anyway: one block per wave
 SCHEDULE_SOFTMAX = (4, 4)
 SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
 SCHEDULE_ATTENTION_BACKWARD = (16, 4)
@@ -168,7 +169,10 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
         shape = batch_a + (num_blocks, BLOCK, BLOCK)
     c = torch.empty(shape, dtype=a.dtype, device=a.device)
 
-    sched = schedule_for(layout, SCHEDULE_SDD) if mode == "sdd" else _group_walk_schedule(layout)
+    if mode == "sdd":
+        sched = schedule_for(layout, SCHEDULE_SDD_F32 if a.dtype == torch.float32 else SCHEDULE_SDD)
+    else:
+        sched = _group_walk_schedule(layout)
     with torch.cuda.device(a.device):
         stream = _k.current_stream()
         ws, ws_bytes = sched.workspace(_k.MODES[mode], batches, size_m, size_n, stream)
