@@ -119,9 +119,11 @@ int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves)
     return slots + groups;   // one record per group in front
 }
 
-int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves, int allow_split, int slice_max,
+int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves, int flags, int slice_max,
                        int slices, int32_t *sched, int64_t capacity, int32_t *counts_out, void *stream)
 {
+    if (flags < 0 || flags > (BSA_SCHED_SPLIT | BSA_SCHED_LONGEST_FIRST))
+        return fail(BSA_ERR_INVALID, "bsa_schedule_build: unknown flags %d", flags);
     if (slice_max < -1 || slice_max > 64)
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: slice_max %d outside [-1, 64]", slice_max);
     if (slice_max >= 0 && slices != 2 && slices != 4)
@@ -134,7 +136,7 @@ int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves, i
     if (capacity < 2 * ((int64_t)groups + 1) + waves + groups || capacity > (1LL << 28))
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: capacity %lld too small for %d groups (use bsa_schedule_capacity)",
                     (long long)capacity, groups);
-    return check_launch(bsa::launch_schedule_build(offsets, groups, cap, waves, allow_split != 0, slice_max, slices, sched, capacity,
+    return check_launch(bsa::launch_schedule_build(offsets, groups, cap, waves, flags, slice_max, slices, sched, capacity,
                                                    counts_out, (hipStream_t)stream),
                         "bsa_schedule_build");
 }

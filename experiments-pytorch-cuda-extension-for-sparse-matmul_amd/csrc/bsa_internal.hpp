@@ -11,7 +11,7 @@ hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_b
                                int32_t *nnz_out, void *workspace, hipStream_t stream);
 
 hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                                 int allow_split, int slice_max, int slices, int32_t *sched, int64_t capacity,
+                                 int flags, int slice_max, int slices, int32_t *sched, int64_t capacity,
                                  int32_t *counts_out, hipStream_t stream);
 
 hipError_t launch_to_sparse(int elem_size, const void *dense, void *sparse, const int32_t *row_blocks,

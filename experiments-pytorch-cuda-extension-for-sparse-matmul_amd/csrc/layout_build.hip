@@ -11,6 +11,7 @@
 // fill the wavefront slots.
 #include "bsa_device.hpp"
 #include "bsa_internal.hpp"
+#include "../../include/bsa.h"
 
 namespace bsa {
 
@@ -124,24 +125,35 @@ __device__ __forceinline__ int waves_of_part(int part_len, int cap, int waves)
 }
 
 __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
-    const int *__restrict__ offsets, int groups, int cap, int waves, int allow_split, int slice_max, int slices,
+    const int *__restrict__ offsets, int groups, int cap, int waves, int flags, int slice_max, int slices,
     int4 *__restrict__ sched, int slot_capacity, int *__restrict__ counts_out)
 {
+    const int allow_split = flags & BSA_SCHED_SPLIT;
+    const bool longest_first = (flags & BSA_SCHED_LONGEST_FIRST) != 0;
     __shared__ int total_slots;
     const int tid = (int)threadIdx.x;
     int4 *meta = sched;
     int4 *slots = sched + groups;
-    // Serial first-fit in three passes.  Row-sliced groups come first and fill whole workgroups of
+    // Serial first-fit in three passes (six with BSA_SCHED_LONGEST_FIRST).  Row-sliced groups come first and fill whole workgroups of
     // their own (their waves need no barrier).  Split groups come next: their parts meet in a
     // workspace after the walk, and workgroups are dispatched in slot order, so starting them first
-    // lets that exchange run while the rest of the launch is still multiplying.  Then the others.
+    // lets that exchange run while the rest of the launch is still multiplying.  Then the others,
+    // in table order or by the length of their longest chunk, longest first: a wave walks its chunk serially, and a
+    // launch of these kernels is only one or two rounds of waves, so a long chunk that starts last
+    // (the late rows of a causal mask) runs on an almost empty machine.
     // A team (the waves of one part) never straddles a workgroup boundary.
     if (tid == 0) {
         int pos = 0, tile_slots = 0, split_groups = 0;
-        for (int pass = 0; pass < 3; ++pass) {
+        constexpr int LEN_CLASSES = 4;     // unsplit groups by their longest chunk: > 3/4, > 1/2, > 1/4 of cap, rest
+        for (int pass = 0; pass < (longest_first ? 2 + LEN_CLASSES : 3); ++pass) {
             for (int g = 0; g < groups; ++g) {
                 const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split, slice_max, slices);
-                const int cls = gp.sliced ? 0 : (gp.parts > 1 ? 1 : 2);
+                int cls = gp.sliced ? 0 : (gp.parts > 1 ? 1 : 2);
+                if (cls == 2 && longest_first) {
+                    const int nw = waves_of_part(gp.len, cap, waves);
+                    const int chunk = (gp.len + nw - 1) / nw;                 // blocks the busiest wave of the team walks
+                    cls = 4 * chunk > 3 * cap ? 2 : (2 * chunk > cap ? 3 : (4 * chunk > cap ? 4 : 5));
+                }
                 if (cls != pass) continue;
                 if (gp.sliced) {
                     meta[g] = make_int4(pos, -1, -1, gp.parts);
@@ -213,10 +225,10 @@ hipError_t launch_layout_build(const uint8_t *mask, int R, int C, int32_t *row_b
 }
 
 hipError_t launch_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                                 int allow_split, int slice_max, int slices, int32_t *sched, int64_t capacity,
+                                 int flags, int slice_max, int slices, int32_t *sched, int64_t capacity,
                                  int32_t *counts_out, hipStream_t stream)
 {
-    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, allow_split, slice_max, slices,
+    schedule_build_kernel<<<1, LB_THREADS, 0, stream>>>(offsets, groups, cap, waves, flags, slice_max, slices,
                                                        (int4 *)sched, (int)(capacity - groups),
                                                        counts_out);
     return hipGetLastError();

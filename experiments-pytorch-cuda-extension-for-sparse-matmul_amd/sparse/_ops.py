@@ -11,8 +11,9 @@ from . import kernel as _k
 
 BLOCK = 32
 # tuning of the wavefront schedules: (target pairs per wavefront, wavefronts per workgroup)
-SCHEDULE_GROUP_WALK = (12, 2)        # groups of at most GROUP_WALK_LONG pairs (rows of attention masks)
-SCHEDULE_GROUP_WALK_LONG = (8, 4)    # tables with longer groups (columns of causal / strided masks)
+# (cap, waves, split long groups, no row slicing, -, longest chunks first)
+SCHEDULE_GROUP_WALK = (12, 2, True, -1, 2, True)        # groups of at most GROUP_WALK_LONG pairs (rows of attention masks)
+SCHEDULE_GROUP_WALK_LONG = (8, 4, True, -1, 2, True)    # tables with longer groups (columns of causal / strided masks)
 GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SDD_F32 = (1, 4)              # fp32 SDD reloads both operands per block anyway: one block per wave
@@ -33,13 +34,14 @@ class Schedule:
     """Device-resident wavefront schedule of one offset table."""
 
     def __init__(self, offsets: torch.Tensor, nnz: int, cap: int, waves: int, allow_split: bool = True,
-                 slice_max: int = -1, slices: int = 2):
+                 slice_max: int = -1, slices: int = 2, longest_first: bool = False):
         groups = offsets.numel() - 1
         capacity = _k.lib.bsa_schedule_capacity(groups, nnz, cap, waves)
         self.table = torch.empty(4 * capacity, dtype=torch.int32, device=offsets.device)
         counts = torch.empty(4, dtype=torch.int32, device=offsets.device)
         with torch.cuda.device(offsets.device):
-            _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves, int(allow_split), slice_max,
+            _k.check(_k.lib.bsa_schedule_build(offsets.data_ptr(), groups, cap, waves,
+                                               int(bool(allow_split)) | (2 if longest_first else 0), slice_max,
                                                slices, self.table.data_ptr(), capacity, counts.data_ptr(),
                                                _k.current_stream()))
         self.workgroups, self.tile_slots, self.split_groups, self.slots = (int(v) for v in counts.tolist())

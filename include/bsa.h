@@ -99,9 +99,14 @@ int bsa_to_dense(int dtype, const void *sparse, void *dense, const uint8_t *mask
 /* ---- wavefront schedule -------------------------------------------------
  * Splits every group of a table into chunks of about `cap` pairs, one chunk
  * per wavefront, and packs the wavefronts into workgroups of `waves`
- * wavefronts.  A group longer than cap * waves pairs is cut into parts of at
- * most that many pairs when `allow_split` != 0 (matmul), and gets longer
- * chunks otherwise (softmax, whose rows cannot be split across workgroups).
+ * wavefronts.  `flags`: with BSA_SCHED_SPLIT a group longer than cap * waves
+ * pairs is cut into parts of at most that many pairs (matmul); without it the
+ * group gets longer chunks (softmax, attention: their rows cannot be split
+ * across workgroups).  With BSA_SCHED_LONGEST_FIRST the groups that are not split
+ * are placed by the length of their longest chunk, longest first, instead of in
+ * table order (a wavefront walks its chunk serially and a launch is only a round
+ * or two of wavefronts, so the long chunks of the late rows of a causal mask would
+ * otherwise start last; it pays for the DSD / DDS walks, not for the others).
  * Empty groups get one wavefront with an empty chunk (it writes the zeros).
  * With `slice_max` >= 0 (softmax only, at most 64) a group of at most slice_max
  * pairs is not chunked at all: it goes whole to `slices` wavefronts (2 or 4),
@@ -119,8 +124,9 @@ int bsa_to_dense(int dtype, const void *sparse, void *dense, const uint8_t *mask
  *                slots, split groups, wavefront slots in use
  */
 int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves);
+enum bsa_sched_flags { BSA_SCHED_SPLIT = 1, BSA_SCHED_LONGEST_FIRST = 2 };
 int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves,
-                       int allow_split, int slice_max, int slices, int32_t *sched,
+                       int flags, int slice_max, int slices, int32_t *sched,
                        int64_t capacity, int32_t *counts_out, void *stream);
 
 /* ---- block-sparse matmul -----------------------------------------------

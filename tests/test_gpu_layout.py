@@ -71,16 +71,17 @@ def test_golden_tables_on_device():
 
 
 @pytest.mark.parametrize("name,mask", _more_masks())
+@pytest.mark.parametrize("longest", [False, True])
 @pytest.mark.parametrize("cap,waves,split", [(4, 8, True), (1, 4, True), (16, 2, True), (3, 1, True),
                                              (4, 8, False), (2, 2, False)])
-def test_schedule_covers_every_pair_once(name, mask, cap, waves, split):
+def test_schedule_covers_every_pair_once(name, mask, cap, waves, split, longest):
     from sparse import _ops
     mask = np.asarray(mask)
     L = _layout(mask)
     for layout in (L.row_layout, L.col_layout):
         offs = layout[1].cpu().numpy()
         groups = len(offs) - 1
-        s = _ops.Schedule(layout[1], layout[0].numel() // 2, cap, waves, split)
+        s = _ops.Schedule(layout[1], layout[0].numel() // 2, cap, waves, split, longest_first=longest)
         raw = s.table.cpu().numpy().reshape(-1, 4)
         meta = raw[:groups]
         tab = raw[groups: groups + s.workgroups * waves]
@@ -114,6 +115,17 @@ def test_schedule_covers_every_pair_once(name, mask, cap, waves, split):
                 if part == parts - 1:
                     assert chunks[-1][2] == offs[g + 1]
         assert np.all(seen[: int(offs[-1])] == 1)
+        if longest:
+            # unsplit groups sit in the order of their longest chunk's class (quarters of cap), longest first
+            classes = []
+            for slot, (g, b, e, team) in enumerate(tab):
+                team = int(team) & 0xFFFFFFFF
+                if g < 0 or (team >> 20) != 1 or slot % waves != (team & 0xF):
+                    continue
+                nw, length = (team >> 4) & 0xF, offs[g + 1] - offs[g]
+                chunk = -(-length // nw)
+                classes.append(0 if 4 * chunk > 3 * cap else 1 if 2 * chunk > cap else 2 if 4 * chunk > cap else 3)
+            assert classes == sorted(classes)
         for g in range(groups):
             length = offs[g + 1] - offs[g]
             want = max(-(-length // (cap * waves)), 1) if split else 1
