@@ -48,7 +48,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; the path shards over batch*heads with no "
-                 "communication, so --gpus N > 1 is not implemented (see DESIGN.md).")
+                 "communication, so --gpus N > 1 is not implemented.")
 
     import torch
     import sparse

@@ -82,26 +82,35 @@ def test_matches_the_unfused_chain_on_config5():
     assert rel_err(to_np(fused[b, h][None]), ref) <= TOL
 
 
-def test_gradients_match_the_unfused_chain():
+@pytest.mark.parametrize("head,causal,name", [(64, True, "rand16"), (64, False, "empty_row_col_6x5"), (128, True, "rand16"),
+                                              (128, False, "long_row_5x40"), (64, True, "long_col_70x3")])
+def test_gradients_match_the_unfused_chain(head, causal, name):
+    """Autograd through sparse.attention (two-launch backward at head dim 64, stored-stack backward at 128)
+    against the chain of the three differentiable operators and against float64 autograd of the dense meaning."""
     import sparse
-    mask = np.asarray(ZOO["rand16"])
+    mask = np.asarray(ZOO[name])
+    rows, cols = mask.shape
     L = sparse.SparseLayout(torch.as_tensor(mask))
-    q, k, v = (t.cuda().requires_grad_(True) for t in _qkv(mask, seed=7))
+    q, k, v = (t.cuda().requires_grad_(True) for t in _qkv(mask, seed=7, head=head))
     g = torch.randn(q.shape, generator=torch.Generator().manual_seed(8)).half().cuda()
-    sparse.attention(q, k, v, L, 0.125, True).backward(g)
+    sparse.attention(q, k, v, L, 0.125, causal).backward(g)
     got = [t.grad.clone() for t in (q, k, v)]
     for t in (q, k, v):
         t.grad = None
     s = sparse.matmul(q, k, "sdd", L, False, True)
-    o = sparse.matmul(sparse.softmax(s, L, 0.125, True), v, "dsd", L)
+    o = sparse.matmul(sparse.softmax(s, L, 0.125, causal), v, "dsd", L)
     o.backward(g)
     for a, t in zip(got, (q, k, v)):
-        assert rel_err(to_np(a), to_np(t.grad)) <= 2e-3
-    # and against float64 autograd of the dense meaning
+        assert rel_err(to_np(a), to_np(t.grad)) <= 4e-3
+    # and against float64 autograd of the dense meaning (rows that see nothing give zeros, not NaN)
     qd, kd, vd = (t.detach().double().cpu().requires_grad_(True) for t in (q, k, v))
-    vis = torch.as_tensor(mask).bool().repeat_interleave(32, 0).repeat_interleave(32, 1) & torch.ones(512, 512).tril().bool()
+    vis = torch.as_tensor(mask).bool().repeat_interleave(32, 0).repeat_interleave(32, 1)
+    if causal:
+        vis = vis & torch.ones(32 * rows, 32 * cols).tril().bool()
     sc = (0.125 * qd @ kd.transpose(-1, -2)).masked_fill(~vis, float("-inf"))
-    (torch.softmax(sc, -1) @ vd).backward(g.double().cpu())
+    p = torch.softmax(sc, -1)
+    p = torch.where(vis.any(-1, keepdim=True), p, torch.zeros_like(p))
+    (p @ vd).backward(g.double().cpu())
     for a, t in zip(got, (qd, kd, vd)):
         assert rel_err(to_np(a), t.grad.numpy()) <= 4e-3
 
