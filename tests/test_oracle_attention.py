@@ -60,3 +60,66 @@ def test_invariants():
     k2[:, 32 * c: 32 * c + 32] += 7.0
     v2[:, 32 * c: 32 * c + 32] -= 3.0
     assert np.allclose(ao.forward(q, k2, v2, hidden, 0.3, False), ao.forward(q, k, v, hidden, 0.3, False))
+
+
+# ---- backward ------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("name,causal", [("known3x3", False), ("known3x3", True), ("empty_row_col_6x5", False), ("rand16", True)])
+def test_backward_equals_the_chain_of_stage_backwards(name, causal):
+    """dq, dk, dv through the three stage oracles (SDD, softmax, DSD and their backward functions)."""
+    mask = np.asarray(ZOO[name])
+    q, k, v = _qkv(mask, d=16, seed=11)
+    dout = np.random.RandomState(12).randn(*q.shape)
+    s = mo.matmul(q, k, "sdd", mask, False, True)
+    p = so.forward(s, mask, 0.2, causal)
+    dp, dv = mo.backward(p, v, dout, "dsd", mask)
+    ds = so.backward(p, dp, mask, 0.2)
+    dq, dk = mo.backward(q, k, ds, "sdd", mask, False, True)
+    for got, want in zip(ao.backward(q, k, v, dout, mask, 0.2, causal), (dq, dk, dv)):
+        assert got.shape == want.shape
+        assert np.max(np.abs(got - want)) <= 1e-11 * max(1.0, np.max(np.abs(want)))
+
+
+def test_backward_by_finite_differences():
+    """Central differences of sum(forward * dout) along random directions of q, k and v."""
+    mask = np.asarray(ZOO["known3x3"])
+    q, k, v = _qkv(mask, d=8, batch=(1,), seed=21)
+    rng = np.random.RandomState(22)
+    dout = rng.randn(*q.shape)
+    grads = ao.backward(q, k, v, dout, mask, 0.3, True)
+    loss = lambda a, b, c: float(np.sum(ao.forward(a, b, c, mask, 0.3, True) * dout))
+    eps = 1e-5
+    for i, g in enumerate(grads):
+        for _ in range(3):
+            d = rng.randn(*g.shape)
+            args_p, args_m = [q, k, v], [q, k, v]
+            args_p[i] = args_p[i] + eps * d
+            args_m[i] = args_m[i] - eps * d
+            numeric = (loss(*args_p) - loss(*args_m)) / (2 * eps)
+            assert abs(numeric - float(np.sum(g * d))) <= 1e-6 * max(1.0, abs(numeric))
+
+
+def test_backward_against_torch_autograd_on_the_dense_meaning():
+    import torch
+    mask = np.asarray(ZOO["rand16"])
+    q, k, v = _qkv(mask, d=8, batch=(1,), seed=31)
+    dout = np.random.RandomState(32).randn(*q.shape)
+    tq, tk, tv = (torch.tensor(t, dtype=torch.float64, requires_grad=True) for t in (q, k, v))
+    vis = torch.as_tensor(mask != 0).repeat_interleave(32, 0).repeat_interleave(32, 1)
+    vis = vis & torch.ones(vis.shape, dtype=torch.bool).tril()
+    s = (0.4 * tq @ tk.transpose(-1, -2)).masked_fill(~vis, float("-inf"))
+    w = torch.softmax(s, -1)
+    w = torch.where(vis.any(-1, keepdim=True), w, torch.zeros_like(w))
+    (w @ tv).backward(torch.tensor(dout))
+    for got, want in zip(ao.backward(q, k, v, dout, mask, 0.4, True), (tq.grad, tk.grad, tv.grad)):
+        assert np.allclose(got, want.numpy(), atol=1e-10)
+
+
+def test_backward_rows_and_columns_without_blocks_get_zero_gradients():
+    mask = np.asarray(ZOO["empty_row_col_6x5"])
+    q, k, v = _qkv(mask, d=8, batch=(1,), seed=41)
+    dq, dk, dv = ao.backward(q, k, v, np.ones_like(q), mask, 1.0, False)
+    empty_rows = np.repeat(~mask.any(axis=1), 32)
+    empty_cols = np.repeat(~mask.any(axis=0), 32)
+    assert empty_rows.any() and empty_cols.any()
+    assert np.all(dq[0, empty_rows] == 0) and np.all(dk[0, empty_cols] == 0) and np.all(dv[0, empty_cols] == 0)
