@@ -51,6 +51,14 @@ class SparseAttention(torch.autograd.Function):
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, layout: SparseLayout, scale: float = 1.0,
               causal: bool = False) -> torch.Tensor:
-    """``softmax(scale * q @ k^T, over the stored blocks of each row) @ v`` for fp16 / bf16
-    ``q [..., 32 R, D]``, ``k``, ``v [..., 32 C, D]``, ``D`` 64 or 128, and an ``R x C`` block layout."""
-    return SparseAttention.apply(q, k, v, layout, scale, causal)
+    """``softmax(scale * q @ k^T, over the stored blocks of each row) @ v`` for ``q [..., 32 R, D]``,
+    ``k``, ``v [..., 32 C, D]`` and an ``R x C`` block layout.  fp16 / bf16 with ``D`` 64 or 128 take the
+    fused kernels; fp32, or another ``D`` (a multiple of 32), is computed as the chain of the three
+    differentiable operators it stands for."""
+    fused = q.dtype in (torch.float16, torch.bfloat16) and q.size(-1) in (64, 128)
+    if fused or not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.float16, torch.bfloat16, torch.float32)):
+        return SparseAttention.apply(q, k, v, layout, scale, causal)     # the fused path also owns the argument checks
+    from .matmul import matmul
+    from .softmax import softmax
+    scores = matmul(q, k, "sdd", layout, False, True)
+    return matmul(softmax(scores, layout, scale, causal), v, "dsd", layout)

@@ -121,11 +121,32 @@ def test_argument_checks():
     L = sparse.SparseLayout(torch.as_tensor(mask))
     q, k, v = (t.cuda() for t in _qkv(mask))
     with pytest.raises(TypeError):
-        sparse.attention(q.float(), k.float(), v.float(), L)
+        sparse.attention(q.float(), k, v, L)                  # mixed dtypes
+    with pytest.raises(TypeError):
+        sparse.attention(q.double(), k.double(), v.double(), L)
     with pytest.raises(ValueError):
         sparse.attention(q[:, :64], k, v, L)
-    with pytest.raises(Exception):
-        sparse.attention(q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous(), L)   # head dim 32
+    with pytest.raises((ValueError, RuntimeError), match="32"):
+        sparse.attention(q[..., :48].contiguous(), k[..., :48].contiguous(), v[..., :48].contiguous(), L)   # not a multiple of 32
+
+
+@pytest.mark.parametrize("dtype,head,causal", [(torch.float32, 64, True), (torch.float32, 96, False), (torch.float16, 32, True),
+                                               (torch.float16, 96, False)])
+def test_other_dtypes_and_head_dims_take_the_chain(dtype, head, causal):
+    """fp32, and head dims the fused kernels are not built for, go through SDD -> softmax -> DSD, with gradients."""
+    import sparse
+    mask = np.asarray(ZOO["rand16"])
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    q, k, v = (t.to(dtype).cuda().requires_grad_(True) for t in _qkv(mask, seed=31, head=head))
+    out = sparse.attention(q, k, v, L, 0.2, causal)
+    assert out.dtype == dtype and out.shape == q.shape
+    qn, kn, vn = (to_np(t.detach().float()) for t in (q, k, v))
+    tol = 1e-5 if dtype == torch.float32 else 2 * TOL
+    assert rel_err(to_np(out.detach().float()), ao.forward(qn, kn, vn, mask, 0.2, causal)) <= tol
+    g = torch.randn(q.shape, generator=torch.Generator().manual_seed(32)).to(dtype).cuda()
+    out.backward(g)
+    for got, want in zip((q.grad, k.grad, v.grad), ao.backward(qn, kn, vn, to_np(g.float()), mask, 0.2, causal)):
+        assert rel_err(to_np(got.float()), want) <= 2 * tol
 
 
 @pytest.mark.parametrize("causal", [False, True])
