@@ -372,7 +372,12 @@ __device__ __forceinline__ bool split_combine(f16v (&acc)[2], const SchedEntry &
     return true;
 }
 
-template <bool S_KC, bool D_KC, bool DSD, int DEPTH, bool BF>
+// FULL: the dense dimension is a multiple of 64, every strip has both 32-wide halves: no per-lane
+// condition on a load and no branch around a product, so the compiler can count the loads in flight
+// (a load under a condition makes it wait for ALL of them before the first use) and can read all six
+// operands of a block from LDS before the first of the four MFMAs instead of exposing the LDS latency
+// four times.
+template <bool S_KC, bool D_KC, bool DSD, int DEPTH, bool BF, bool FULL>
 __global__ __launch_bounds__(512) void gw_f16_kernel(
     const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
     const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
@@ -389,7 +394,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     const SchedEntry e = sched[swg * W + w];
     if (BSA_ABLATE(64)) { if (e.group == 12345678) out[0] = (half_t)1; return; }
     const int y0 = 64 * (int)blockIdx.y;
-    const int ytiles = (DN - y0) >= 64 ? 2 : 1;
+    const int ytiles = FULL ? 2 : ((DN - y0) >= 64 ? 2 : 1);
 
     half_t *tile_s = reinterpret_cast<half_t *>(lds_raw + (size_t)w * GW_LDS_PER_WAVE);
     half_t *tile_d = tile_s + BS2;
@@ -418,7 +423,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
                 int cidx = l + 64 * q;
                 int row = cidx >> 3, ch = cidx & 7;
                 uint4 v = make_uint4(0, 0, 0, 0);
-                if (ch < pieces) v = ldg16(src + (size_t)row * DN + 8 * ch);
+                if (FULL || ch < pieces) v = ldg16(src + (size_t)row * DN + 8 * ch);
                 (q < 2 ? f.d0[q & 1] : f.d1[q & 1]) = v;
             }
         }
@@ -443,18 +448,20 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
             lds_put_strip(tile_d, f.d0, f.d1);
         }
         wave_lds_fence();
+        h8 sop[2], dop[2][2];
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            const h8 sop = S_KC ? lds_get_kc(tile_s, s) : lds_get_ks<!DSD>(tile_s, s);
+            sop[s] = S_KC ? lds_get_kc(tile_s, s) : lds_get_ks<!DSD>(tile_s, s);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (t < ytiles) {
-                    const h8 dop = D_KC ? lds_get_kc(tile_d + t * BS2, s)
-                                        : lds_get_strip<DSD>(tile_d, 32 * t, s);
-                    acc[t] = DSD ? mfma_16<BF>(dop, sop, acc[t]) : mfma_16<BF>(sop, dop, acc[t]);
-                }
-            }
+            for (int t = 0; t < 2; ++t)
+                if (t < ytiles)
+                    dop[s][t] = D_KC ? lds_get_kc(tile_d + t * BS2, s) : lds_get_strip<DSD>(tile_d, 32 * t, s);
         }
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                if (t < ytiles) acc[t] = DSD ? mfma_16<BF>(dop[s][t], sop[s], acc[t]) : mfma_16<BF>(sop[s], dop[s][t], acc[t]);
     };
 
     BSA_TRACE_MARK_NOWAIT(1)
@@ -464,11 +471,25 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
             const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
             win.fetch(blocks, seg, seg_end);
             if (BSA_ABLATE(128)) { if (win.idx == 12345678) out[0] = (half_t)1; return; }
+            int p = seg;
+            if (seg_end - seg >= 2 * DEPTH) {
+                // long enough for a steady state in which every load is unconditional
 #pragma unroll
-            for (int d = 0; d < DEPTH; ++d)
-                if (seg + d < seg_end) load(seg + d, fr[d]);
+                for (int d = 0; d < DEPTH; ++d) load(seg + d, fr[d]);
+                for (; p + 2 * DEPTH <= seg_end; p += DEPTH) {
+#pragma unroll
+                    for (int d = 0; d < DEPTH; ++d) {
+                        compute(fr[d]);
+                        load(p + d + DEPTH, fr[d]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int d = 0; d < DEPTH; ++d)
+                    if (seg + d < seg_end) load(seg + d, fr[d]);
+            }
             BSA_TRACE_MARK_NOWAIT(2)
-            for (int p = seg; p < seg_end; p += DEPTH) {
+            for (; p < seg_end; p += DEPTH) {                // the last pairs: loads only while pairs are left
 #pragma unroll
                 for (int d = 0; d < DEPTH; ++d) {
                     if (p + d < seg_end) {
@@ -620,15 +641,17 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
     ws.split_groups = p.split_groups;
     ws.counters = (int *)p.workspace;
     ws.tiles = (float *)((char *)p.workspace + gw_counter_bytes(p.split_groups, p.batches, DN));
-    if (dtype == BSA_F16)
-        gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false><<<grid, block, lds, st>>>(
-            (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
-            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
-    else if (dtype == BSA_BF16)
-        gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, true><<<grid, block, lds, st>>>(
-            (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks,
-            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
-    else
+#define BSA_GW_ARGS (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks, \
+                    sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0
+    const bool full = DN % 64 == 0;
+    if (dtype == BSA_F16) {
+        if (full) gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false, true><<<grid, block, lds, st>>>(BSA_GW_ARGS);
+        else gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false, false><<<grid, block, lds, st>>>(BSA_GW_ARGS);
+    } else if (dtype == BSA_BF16) {
+        if (full) gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, true, true><<<grid, block, lds, st>>>(BSA_GW_ARGS);
+        else gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, true, false><<<grid, block, lds, st>>>(BSA_GW_ARGS);
+    } else
+#undef BSA_GW_ARGS
         gw_f32_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(
             (const float *)sp, (const float *)dn, (float *)p.c, (const BlockDesc *)p.blocks,
             sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
