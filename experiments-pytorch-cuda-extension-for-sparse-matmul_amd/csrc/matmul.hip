@@ -138,36 +138,52 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
             aop[kb][1] = get_a(tile_a, 1);
         }
         uint4 braw[2][KB][2];
-        BlockDesc d[2];
         DescWindow win;
+        auto load_tiles = [&](int p, uint4 (&raw)[KB][2]) {
+            const int cblk = win.get(p).col();
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) load_b(cblk, kb, raw[kb]);
+        };
+        auto multiply = [&](int p, const uint4 (&raw)[KB][2]) {
+            wave_lds_fence();
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) put_b(tile_b + kb * BS2, raw[kb]);
+            wave_lds_fence();
+            h8 bop[KB][2];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                bop[kb][0] = get_b(tile_b + kb * BS2, 0);
+                bop[kb][1] = get_b(tile_b + kb * BS2, 1);
+            }
+            f16v acc = {0};
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                acc = mfma_16<BF>(bop[kb][0], aop[kb][0], acc);
+                acc = mfma_16<BF>(bop[kb][1], aop[kb][1], acc);
+            }
+            store(win.get(p).idx, acc);
+        };
+        // One block ahead: the tiles of block p + 1 are requested before block p is multiplied.  A load
+        // under a condition makes the compiler wait for every load and store in flight before the next
+        // use, which would cancel the prefetch, so the loop body holds none; the last one or two blocks
+        // of a segment are straight-line code.
         for (int seg = e.begin; seg < e.end; seg += WAVE) {
             const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
             win.fetch(blocks, seg, seg_end);
-            d[0] = win.get(seg);
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) load_b(d[0].col(), kb, braw[0][kb]);
-            for (int p = seg; p < seg_end; p += 2) {
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    if (p + u < seg_end) {
-                        if (p + u + 1 < seg_end) {
-                            d[u ^ 1] = win.get(p + u + 1);
-#pragma unroll
-                            for (int kb = 0; kb < KB; ++kb) load_b(d[u ^ 1].col(), kb, braw[u ^ 1][kb]);
-                        }
-                        wave_lds_fence();
-#pragma unroll
-                        for (int kb = 0; kb < KB; ++kb) put_b(tile_b + kb * BS2, braw[u][kb]);
-                        wave_lds_fence();
-                        f16v acc = {0};
-#pragma unroll
-                        for (int kb = 0; kb < KB; ++kb) {
-                            acc = mfma_16<BF>(get_b(tile_b + kb * BS2, 0), aop[kb][0], acc);
-                            acc = mfma_16<BF>(get_b(tile_b + kb * BS2, 1), aop[kb][1], acc);
-                        }
-                        store(d[u].idx, acc);
-                    }
-                }
+            load_tiles(seg, braw[0]);
+            int p = seg;
+            for (; p + 2 < seg_end; p += 2) {
+                load_tiles(p + 1, braw[1]);
+                multiply(p, braw[0]);
+                load_tiles(p + 2, braw[0]);
+                multiply(p + 1, braw[1]);
+            }
+            if (p + 1 < seg_end) {
+                load_tiles(p + 1, braw[1]);
+                multiply(p, braw[0]);
+                multiply(p + 1, braw[1]);
+            } else {
+                multiply(p, braw[0]);
             }
         }
     } else {
