@@ -13,7 +13,7 @@ BLOCK = 32
 # tuning of the wavefront schedules: (target pairs per wavefront, wavefronts per workgroup)
 # (cap, waves, split long groups, no row slicing, -, longest chunks first)
 SCHEDULE_GROUP_WALK = (12, 2, True, -1, 2, True)        # groups of at most GROUP_WALK_LONG pairs (rows of attention masks)
-SCHEDULE_GROUP_WALK_LONG = (8, 4, True, -1, 2, True)    # tables with longer groups (columns of causal / strided masks)
+SCHEDULE_GROUP_WALK_LONG = (10, 4, True, -1, 2, True)    # tables with longer groups (columns of causal / strided masks)
 GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SDD_F32 = (1, 4)              # fp32 SDD reloads both operands per block anyway: one block per wave
