@@ -13,7 +13,10 @@
 // measured at a third of the coalesced rate and are only used by the fp32
 // kernels.  Data touched once (sparse blocks, results) moves with non-temporal
 // loads and stores; dense tiles, which are re-read out of L2, do not.  No
-// workgroup barrier sits in any inner loop.
+// workgroup barrier sits in any inner loop, and no load under a condition sits
+// in the steady state of a block loop (tails are peeled): behind a conditional
+// load the compiler can no longer count the loads in flight and waits for all of
+// them, which cancels the prefetch.
 //
 // Work distribution: a schedule (see bsa.h) hands every wavefront a chunk of
 // consecutive table pairs of one group.  SDD: the chunk's blocks share the
