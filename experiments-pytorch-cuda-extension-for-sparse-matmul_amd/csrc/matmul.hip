@@ -129,19 +129,17 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
 
     if (KBT > 0) {
         constexpr int KB = KBT > 0 ? KBT : 1;
+        // The wave's first requests all go out together: its block descriptors, the A tiles of every
+        // k-block, then (as soon as the descriptors are back) the B tiles of its first block; the A tiles
+        // are turned into operand registers while those are in flight.  One memory round trip instead
+        // of one per k-block plus one for the descriptors plus one for the first block.
         h8 aop[KB][2];
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-            uint4 raw[2];
-            load_a(kb, raw);
-            wave_lds_fence();
-            put_a(tile_a, raw);
-            wave_lds_fence();
-            aop[kb][0] = get_a(tile_a, 0);
-            aop[kb][1] = get_a(tile_a, 1);
-        }
-        uint4 braw[2][KB][2];
+        uint4 araw[KB][2], braw[2][KB][2];
         DescWindow win;
+        const int first_end = e.begin + WAVE < e.end ? e.begin + WAVE : e.end;
+        win.fetch(blocks, e.begin, first_end);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) load_a(kb, araw[kb]);
         auto load_tiles = [&](int p, uint4 (&raw)[KB][2]) {
             const int cblk = win.get(p).col();
 #pragma unroll
@@ -170,10 +168,21 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
         // under a condition makes the compiler wait for every load and store in flight before the next
         // use, which would cancel the prefetch, so the loop body holds none; the last one or two blocks
         // of a segment are straight-line code.
+        load_tiles(e.begin, braw[0]);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            wave_lds_fence();
+            put_a(tile_a, araw[kb]);
+            wave_lds_fence();
+            aop[kb][0] = get_a(tile_a, 0);
+            aop[kb][1] = get_a(tile_a, 1);
+        }
         for (int seg = e.begin; seg < e.end; seg += WAVE) {
             const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
-            win.fetch(blocks, seg, seg_end);
-            load_tiles(seg, braw[0]);
+            if (seg != e.begin) {
+                win.fetch(blocks, seg, seg_end);
+                load_tiles(seg, braw[0]);
+            }
             int p = seg;
             for (; p + 2 < seg_end; p += 2) {
                 load_tiles(p + 1, braw[1]);
