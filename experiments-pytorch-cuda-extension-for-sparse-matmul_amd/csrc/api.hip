@@ -211,6 +211,7 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
 
     bsa::MatmulArgs p{a, b, c, blocks, sched, groups, sched_wgs, sched_waves, sched_tile_slots, sched_split_groups,
                       workspace, nnz, batches, M, N, K, tr_a != 0, tr_b != 0, sparse_batches != batches};
+    p.row_table = row_table;
     if (nnz == 0 && mode == BSA_SDD) return BSA_OK;   // nothing to write
     hipError_t err = mode == BSA_SDD ? bsa::launch_sdd(dtype, p, (hipStream_t)stream)
                                      : bsa::launch_group_walk(dtype, mode == BSA_DSD, p, (hipStream_t)stream);

@@ -32,6 +32,7 @@ struct MatmulArgs {
     int M, N, K;
     bool tr_a, tr_b;
     bool sparse_shared;   // DSD / DDS: the sparse operand has no batch dimension
+    bool row_table = false;   // DSD / DDS: `blocks` is the row-major table, whose pair p names block p
 };
 
 hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t stream);

@@ -410,7 +410,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
     const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
     const SchedEntry *__restrict__ sched, SplitWorkspace ws,
-    int n_swg, int batches, int nnz, int DN, int KT, int XT, int sp_shared)
+    int n_swg, int batches, int nnz, int DN, int KT, int XT, int sp_shared, int idx_is_pos)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     BSA_TRACE_BEGIN
@@ -434,10 +434,9 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     struct Frag { uint4 s[2]; uint4 d0[2]; uint4 d1[2]; };
 
     DescWindow win;
-    auto load = [&](int p, Frag &f) {
+    auto load_dense = [&](int p, Frag &f) {
         const BlockDesc d = win.get(p);
         const int kblk = S_KC ? d.col() : d.row();
-        if (!BSA_ABLATE(4)) ldg_block32_stream(spb + (size_t)d.idx * BS2, f.s);
         if (BSA_ABLATE(2)) return;
         if (D_KC) {          // stored [DN][KT]: two 32 x 32 tiles, rows KT apart
             const half_t *src = dnb + (size_t)y0 * KT + BS * kblk;
@@ -455,6 +454,10 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
                 (q < 2 ? f.d0[q & 1] : f.d1[q & 1]) = v;
             }
         }
+    };
+    auto load = [&](int p, Frag &f) {
+        if (!BSA_ABLATE(4)) ldg_block32_stream(spb + (size_t)win.get(p).idx * BS2, f.s);
+        load_dense(p, f);
     };
 
     f16v acc[2] = {{0}, {0}};
@@ -501,9 +504,17 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
             if (BSA_ABLATE(128)) { if (win.idx == 12345678) out[0] = (half_t)1; return; }
             int p = seg;
             if (seg_end - seg >= 2 * DEPTH) {
-                // long enough for a steady state in which every load is unconditional
+                // long enough for a steady state in which every load is unconditional.
+                // In a row-major table pair p names block p, so the first block (from HBM, the longest
+                // wait of the wave) is requested without waiting for the descriptors just asked for.
+                if (idx_is_pos) {
+                    if (!BSA_ABLATE(4)) ldg_block32_stream(spb + (size_t)seg * BS2, fr[0].s);
+                    load_dense(seg, fr[0]);
+                } else {
+                    load(seg, fr[0]);
+                }
 #pragma unroll
-                for (int d = 0; d < DEPTH; ++d) load(seg + d, fr[d]);
+                for (int d = 1; d < DEPTH; ++d) load(seg + d, fr[d]);
                 for (; p + 2 * DEPTH <= seg_end; p += DEPTH) {
 #pragma unroll
                     for (int d = 0; d < DEPTH; ++d) {
@@ -670,7 +681,8 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
     ws.counters = (int *)p.workspace;
     ws.tiles = (float *)((char *)p.workspace + gw_counter_bytes(p.split_groups, p.batches, DN));
 #define BSA_GW_ARGS (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks, \
-                    sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0
+                    sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0, \
+                    p.row_table ? 1 : 0
     const bool full = DN % 64 == 0;
     if (dtype == BSA_F16) {
         if (full) gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false, true><<<grid, block, lds, st>>>(BSA_GW_ARGS);
