@@ -654,6 +654,12 @@ hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t st)
                     32 * p.mask_rows, 32 * p.mask_cols, p.scale * 1.4426950408889634f, p.causal ? 1 : 0
     const size_t lds = (size_t)p.sched_waves * at_lds_per_wave(p.head_dim);
     if (p.head_dim == 64) {
+        if (lds > 65536) {   // 8 waves x 8.5 KB
+            const void *fn = p.bf16 ? (const void *)attention_fwd_f16_kernel<64, true>
+                                    : (const void *)attention_fwd_f16_kernel<64, false>;
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
         if (p.bf16) attention_fwd_f16_kernel<64, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
         else attention_fwd_f16_kernel<64, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
     } else {

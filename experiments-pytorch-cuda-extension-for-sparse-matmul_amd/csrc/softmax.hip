@@ -32,6 +32,7 @@ __device__ int g_sm_ablate = 0;   // debug builds: 8 = no stores, 16 = no loads
 #endif
 
 constexpr int SM_MAX_WAVES = 8;
+constexpr int SM_STREAM_REGS = 16;  // 16-byte registers a batch of the streaming walks (rows too long for registers) may hold
 
 template <typename T> struct Chunk;
 template <> struct Chunk<half_t> {
@@ -495,6 +496,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
     typedef Chunk<T> C;
     constexpr int NQ = C::NQ, EPC = C::EPC, LPR = C::LPR;
     constexpr int ROWS_PER_Q = WAVE / LPR;
+    constexpr int SM_STREAM = SM_STREAM_REGS / NQ;            // blocks per batch: 8 (16-bit types) or 4; divides 64
     __shared__ float2 stats[SM_MAX_WAVES][BS];
 
     int batch, swg;
@@ -566,26 +568,39 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
             }
         }
     } else if (active) {
-        // streaming pass 1: online max / sum
-        for (int p = e.begin; p < e.end; ++p) {
-            if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
-            const BlockDesc d = win.get(p);
-            const T *src = xb + (size_t)d.idx * BS2;
+        // Streaming pass 1: online max / sum, SM_STREAM blocks at a time.  All loads of a batch go out
+        // before the first block is touched (one memory latency per batch instead of one per block;
+        // a batch past the end of the chunk reloads the last block, so no load sits under a condition).
+        for (int p0 = e.begin; p0 < e.end; p0 += SM_STREAM) {
+            if (p0 > e.begin && ((p0 - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p0, e.end);
+            uint4 rs[SM_STREAM][NQ];
+            int cs[SM_STREAM];
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-                float v[EPC];
-                scaled_chunk<T>(ldg16_stream(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
-                                scale2, causal, v);
-                float bm = v[0];
+            for (int j = 0; j < SM_STREAM; ++j) {
+                const BlockDesc d = win.get(p0 + j < e.end ? p0 + j : e.end - 1);
+                cs[j] = d.col();
+                const T *src = xb + (size_t)d.idx * BS2;
 #pragma unroll
-                for (int i = 1; i < EPC; ++i) bm = fmaxf(bm, v[i]);
-                const float nm = fmaxf(m[q], bm);
-                const float mm = finite_or_zero(nm);
-                float acc = s[q] * exp2_fast(m[q] - mm);
+                for (int q = 0; q < NQ; ++q) rs[j][q] = ldg16_stream(src + (l + WAVE * q) * EPC);
+            }
 #pragma unroll
-                for (int i = 0; i < EPC; ++i) acc += exp2_fast(v[i] - mm);
-                s[q] = acc;
-                m[q] = nm;
+            for (int j = 0; j < SM_STREAM; ++j) {
+                if (p0 + j >= e.end) break;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    float v[EPC];
+                    scaled_chunk<T>(rs[j][q], row0 + q * ROWS_PER_Q, col0, cs[j], e.group, scale2, causal, v);
+                    float bm = v[0];
+#pragma unroll
+                    for (int i = 1; i < EPC; ++i) bm = fmaxf(bm, v[i]);
+                    const float nm = fmaxf(m[q], bm);
+                    const float mm = finite_or_zero(nm);
+                    float acc = s[q] * exp2_fast(m[q] - mm);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) acc += exp2_fast(v[i] - mm);
+                    s[q] = acc;
+                    m[q] = nm;
+                }
             }
         }
         // lanes of a row hold different (m, s): bring them to the row max
@@ -645,20 +660,32 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
             }
         }
     } else {
-        // streaming pass 2: re-read, normalise, write
-        for (int p = e.begin; p < e.end; ++p) {
-            if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
-            const BlockDesc d = win.get(p);
-            const T *src = xb + (size_t)d.idx * BS2;
-            T *dst = yb + (size_t)d.idx * BS2;
+        // streaming pass 2: re-read, normalise, write, in the same batches
+        for (int p0 = e.begin; p0 < e.end; p0 += SM_STREAM) {
+            if (((p0 - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p0, e.end);
+            uint4 rs[SM_STREAM][NQ];
+            int cs[SM_STREAM], is[SM_STREAM];
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-                float v[EPC];
-                scaled_chunk<T>(ldg16_stream(src + (l + WAVE * q) * EPC), row0 + q * ROWS_PER_Q, col0, d.col(), e.group,
-                                scale2, causal, v);
+            for (int j = 0; j < SM_STREAM; ++j) {
+                const BlockDesc d = win.get(p0 + j < e.end ? p0 + j : e.end - 1);
+                cs[j] = d.col();
+                is[j] = d.idx;
+                const T *src = xb + (size_t)d.idx * BS2;
 #pragma unroll
-                for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - gm[q]) * inv_s[q];
-                stg16_stream(dst + (l + WAVE * q) * EPC, C::pack(v));
+                for (int q = 0; q < NQ; ++q) rs[j][q] = ldg16_stream(src + (l + WAVE * q) * EPC);
+            }
+#pragma unroll
+            for (int j = 0; j < SM_STREAM; ++j) {
+                if (p0 + j >= e.end) break;
+                T *dst = yb + (size_t)is[j] * BS2;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    float v[EPC];
+                    scaled_chunk<T>(rs[j][q], row0 + q * ROWS_PER_Q, col0, cs[j], e.group, scale2, causal, v);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) v[i] = exp2_fast(v[i] - gm[q]) * inv_s[q];
+                    stg16_stream(dst + (l + WAVE * q) * EPC, C::pack(v));
+                }
             }
         }
     }
@@ -791,6 +818,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
     typedef Chunk<T> C;
     constexpr int NQ = C::NQ, EPC = C::EPC, LPR = C::LPR;
     constexpr int ROWS_PER_Q = WAVE / LPR;
+    constexpr int SM_STREAM_BWD = SM_STREAM_REGS / (2 * NQ);  // two operands per block: 4 or 2 blocks per batch
     __shared__ float dots[SM_MAX_WAVES][BS];
 
     int batch, swg;
@@ -845,16 +873,30 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
             }
         }
     } else if (active) {
-        for (int p = e.begin; p < e.end; ++p) {
-            if (p > e.begin && ((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
-            const size_t o = boff + (size_t)win.get(p).idx * BS2;
+        // streaming, SM_STREAM_BWD blocks at a time: all loads of a batch go out before the first use
+        for (int p0 = e.begin; p0 < e.end; p0 += SM_STREAM_BWD) {
+            if (p0 > e.begin && ((p0 - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p0, e.end);
+            uint4 sy[SM_STREAM_BWD][NQ], sd[SM_STREAM_BWD][NQ];
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-                float a[EPC], b[EPC];
-                C::unpack(ldg16_stream(y + o + (l + WAVE * q) * EPC), a);
-                C::unpack(ldg16_stream(dy + o + (l + WAVE * q) * EPC), b);
+            for (int j = 0; j < SM_STREAM_BWD; ++j) {
+                const size_t o = boff + (size_t)win.get(p0 + j < e.end ? p0 + j : e.end - 1).idx * BS2;
 #pragma unroll
-                for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
+                for (int q = 0; q < NQ; ++q) {
+                    sy[j][q] = ldg16_stream(y + o + (l + WAVE * q) * EPC);
+                    sd[j][q] = ldg16_stream(dy + o + (l + WAVE * q) * EPC);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < SM_STREAM_BWD; ++j) {
+                if (p0 + j >= e.end) break;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    float a[EPC], b[EPC];
+                    C::unpack(sy[j][q], a);
+                    C::unpack(sd[j][q], b);
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) dot[q] += a[i] * b[i];
+                }
             }
         }
     }
@@ -895,13 +937,25 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
             }
         }
     } else {
-        for (int p = e.begin; p < e.end; ++p) {
-            if (((p - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p, e.end);
-            const size_t o = boff + (size_t)win.get(p).idx * BS2;
+        for (int p0 = e.begin; p0 < e.end; p0 += SM_STREAM_BWD) {
+            if (((p0 - e.begin) & (WAVE - 1)) == 0) win.fetch(blocks, p0, e.end);
+            uint4 sy[SM_STREAM_BWD][NQ], sd[SM_STREAM_BWD][NQ];
+            size_t os[SM_STREAM_BWD];
 #pragma unroll
-            for (int q = 0; q < NQ; ++q)
-                stg16_stream(dx + o + (l + WAVE * q) * EPC,
-                      finish(ldg16_stream(y + o + (l + WAVE * q) * EPC), ldg16_stream(dy + o + (l + WAVE * q) * EPC), q));
+            for (int j = 0; j < SM_STREAM_BWD; ++j) {
+                os[j] = boff + (size_t)win.get(p0 + j < e.end ? p0 + j : e.end - 1).idx * BS2;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    sy[j][q] = ldg16_stream(y + os[j] + (l + WAVE * q) * EPC);
+                    sd[j][q] = ldg16_stream(dy + os[j] + (l + WAVE * q) * EPC);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < SM_STREAM_BWD; ++j) {
+                if (p0 + j >= e.end) break;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) stg16_stream(dx + os[j] + (l + WAVE * q) * EPC, finish(sy[j][q], sd[j][q], q));
+            }
         }
     }
 }

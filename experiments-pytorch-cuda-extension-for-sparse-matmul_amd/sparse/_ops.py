@@ -18,6 +18,8 @@ GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SDD_F32 = (1, 4)              # fp32 SDD reloads both operands per block anyway: one block per wave
 SCHEDULE_SOFTMAX = (4, 4)
+SOFTMAX_WAVES_LONG_ROWS = 8
+ATTENTION_WAVES_LONG_GROUPS = 8
 SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
 SCHEDULE_ATTENTION_BACKWARD = (16, 4)
 SCHEDULE_ATTENTION_BACKWARD_COLUMNS = (8, 8)
@@ -93,10 +95,24 @@ def _group_walk_schedule(layout):
     return schedule_for(layout, kind)
 
 
+def _attention_schedule(layout, kind):
+    """Schedule of a fused attention walk: a group is never split across workgroups there, so a table
+    with a group longer than the workgroup's share gets the most waves a workgroup holds."""
+    cap, waves = kind
+    if _longest_group(layout[1]) > cap * waves:
+        waves = ATTENTION_WAVES_LONG_GROUPS
+    return schedule_for(layout, (cap, waves, False))
+
+
 def _softmax_schedule(layout, dtype, backward):
     cap, waves = SCHEDULE_SOFTMAX
     which = 1 if backward else 0
-    return schedule_for(layout, (cap, waves, False, SOFTMAX_SLICE_MAX[dtype][which], SOFTMAX_SLICES[which]))
+    slice_max = SOFTMAX_SLICE_MAX[dtype][which]
+    if _longest_group(layout[1]) > slice_max:
+        # a row too long for the register-resident walk is streamed by the waves of ONE workgroup (a row
+        # cannot be split across workgroups): as many waves as a workgroup holds keep its chunks short
+        waves = SOFTMAX_WAVES_LONG_ROWS
+    return schedule_for(layout, (cap, waves, False, slice_max, SOFTMAX_SLICES[which]))
 
 
 def _check_layout(layout, name):
@@ -277,8 +293,7 @@ def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=F
     out = torch.empty_like(q)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device) if return_lse else None
     if out.numel() > 0:
-        cap, waves = SCHEDULE_ATTENTION
-        sched = schedule_for(row_layout, (cap, waves, False))
+        sched = _attention_schedule(row_layout, SCHEDULE_ATTENTION)
         with torch.cuda.device(q.device):
             _k.check(_k.lib.bsa_attention_forward(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
@@ -306,8 +321,7 @@ def sparse_attention_backward_scores(q, k, v, dout, out, lse, row_blocks, row_ta
     ds = torch.empty(shape, dtype=q.dtype, device=q.device)
     dq = torch.empty_like(q) if with_dq else None
     if q.numel() > 0:
-        cap, waves = SCHEDULE_ATTENTION_BACKWARD
-        sched = schedule_for(row_layout, (cap, waves, False))
+        sched = _attention_schedule(row_layout, SCHEDULE_ATTENTION_BACKWARD)
         with torch.cuda.device(q.device):
             _k.check(_k.lib.bsa_attention_backward_scores(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
@@ -338,8 +352,8 @@ def sparse_attention_backward(q, k, v, dout, out, lse, row_blocks, row_table, co
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     if q.numel() > 0:
         delta = torch.empty_like(lse)
-        rs = schedule_for(row_layout, SCHEDULE_ATTENTION_BACKWARD + (False,))
-        cs = schedule_for(col_layout, SCHEDULE_ATTENTION_BACKWARD_COLUMNS + (False,))
+        rs = _attention_schedule(row_layout, SCHEDULE_ATTENTION_BACKWARD)
+        cs = _attention_schedule(col_layout, SCHEDULE_ATTENTION_BACKWARD_COLUMNS)
         with torch.cuda.device(q.device):
             _k.check(_k.lib.bsa_attention_backward(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
