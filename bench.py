@@ -318,11 +318,17 @@ def main():
                    nbytes=(4 * 8192 * 64 + 4 * n5 * 1024) * b5 * 2)
         run_config("config5_fused_attention", lambda: sparse.attention(c5["q"], c5["k"], c5["v"], l5, 0.125, False), 4,
                    flops=f5, nbytes=4 * 8192 * 64 * b5 * 2)
-        sc5 = sparse.matmul(c5["q"], c5["k"], "sdd", l5, False, True)
-        run_config("config5_softmax_alone", lambda: sparse.softmax(sc5, l5, 0.125, False), 4,
-                   nbytes=2 * n5 * 1024 * b5 * 2)
+        with torch.no_grad():
+            sc5 = sparse.matmul(c5["q"], c5["k"], "sdd", l5, False, True)
+            p5 = sparse.softmax(sc5, l5, 0.125, False)
+        blk5, dense5 = n5 * 1024 * b5 * 2, 8192 * 64 * b5 * 2
+        run_config("config5_sdd_alone", lambda: sparse.matmul(c5["q"], c5["k"], "sdd", l5, False, True), 4,
+                   flops=f5 / 2, nbytes=2 * dense5 + blk5)
+        run_config("config5_softmax_alone", lambda: sparse.softmax(sc5, l5, 0.125, False), 4, nbytes=2 * blk5)
+        run_config("config5_dsd_alone", lambda: sparse.matmul(p5, c5["v"], "dsd", l5), 4,
+                   flops=f5 / 2, nbytes=blk5 + 2 * dense5)
         configs["config5_nnz"] = n5
-        del c5, sc5
+        del c5, sc5, p5
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/): same
     # workload, same kernels; absent file -> null
