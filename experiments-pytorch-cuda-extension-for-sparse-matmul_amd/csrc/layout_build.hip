@@ -134,25 +134,42 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
     const int tid = (int)threadIdx.x;
     int4 *meta = sched;
     int4 *slots = sched + groups;
-    // Serial first-fit in three passes (six with BSA_SCHED_LONGEST_FIRST).  Row-sliced groups come first and fill whole workgroups of
+    // Serial first-fit in three passes (nine with BSA_SCHED_LONGEST_FIRST).  Row-sliced groups come first and fill whole workgroups of
     // their own (their waves need no barrier).  Split groups come next: their parts meet in a
     // workspace after the walk, and workgroups are dispatched in slot order, so starting them first
-    // lets that exchange run while the rest of the launch is still multiplying.  Then the others,
-    // in table order or by the length of their longest chunk, longest first: a wave walks its chunk serially, and a
-    // launch of these kernels is only one or two rounds of waves, so a long chunk that starts last
-    // (the late rows of a causal mask) runs on an almost empty machine.
+    // lets that exchange run while the rest of the launch is still multiplying.  Then the others.
+    // Within the sliced and within the unsplit groups the order is table order, or, longest first, by
+    // length (sliced: quarters of the longest sliced group; unsplit: the longest chunk in quarters of
+    // cap): a wave walks its chunk serially and a launch of these kernels is only one or two rounds of
+    // waves, so a long chunk that starts last (the late rows of a causal mask) runs on an almost empty machine.
     // A team (the waves of one part) never straddles a workgroup boundary.
     if (tid == 0) {
         int pos = 0, tile_slots = 0, split_groups = 0;
-        constexpr int LEN_CLASSES = 4;     // unsplit groups by their longest chunk: > 3/4, > 1/2, > 1/4 of cap, rest
-        for (int pass = 0; pass < (longest_first ? 2 + LEN_CLASSES : 3); ++pass) {
+        constexpr int LEN_CLASSES = 4;     // by length: > 3/4, > 1/2, > 1/4 of the yardstick, rest
+        const int sliced_passes = longest_first ? LEN_CLASSES : 1;
+        int longest_sliced = 0;
+        if (longest_first)
+            for (int g = 0; g < groups; ++g) {
+                const int len = offsets[g + 1] - offsets[g];
+                if (len <= slice_max && len > longest_sliced) longest_sliced = len;
+            }
+        auto len_class = [](int len, int yard) {
+            return 4 * len > 3 * yard ? 0 : (2 * len > yard ? 1 : (4 * len > yard ? 2 : 3));
+        };
+        for (int pass = 0; pass < sliced_passes + (longest_first ? 1 + LEN_CLASSES : 2); ++pass) {
             for (int g = 0; g < groups; ++g) {
                 const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split, slice_max, slices);
-                int cls = gp.sliced ? 0 : (gp.parts > 1 ? 1 : 2);
-                if (cls == 2 && longest_first) {
-                    const int nw = waves_of_part(gp.len, cap, waves);
-                    const int chunk = (gp.len + nw - 1) / nw;                 // blocks the busiest wave of the team walks
-                    cls = 4 * chunk > 3 * cap ? 2 : (2 * chunk > cap ? 3 : (4 * chunk > cap ? 4 : 5));
+                int cls;
+                if (gp.sliced) {
+                    cls = longest_first ? len_class(gp.len, longest_sliced) : 0;
+                } else if (gp.parts > 1) {
+                    cls = sliced_passes;
+                } else {
+                    cls = sliced_passes + 1;
+                    if (longest_first) {
+                        const int nw = waves_of_part(gp.len, cap, waves);
+                        cls += len_class((gp.len + nw - 1) / nw, cap);   // blocks the busiest wave of the team walks
+                    }
                 }
                 if (cls != pass) continue;
                 if (gp.sliced) {
@@ -173,7 +190,7 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
                 meta[g] = make_int4(first, split ? tile_slots : -1, split ? split_groups : -1, gp.parts);
                 if (split) { tile_slots += gp.parts; split_groups += 1; }
             }
-            if (pass == 0) pos = (pos + waves - 1) / waves * waves;
+            if (pass == sliced_passes - 1) pos = (pos + waves - 1) / waves * waves;
         }
         int n_wgs = (pos + waves - 1) / waves;
         total_slots = n_wgs * waves;

@@ -18,6 +18,7 @@ GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
 SCHEDULE_SDD_F32 = (1, 4)              # fp32 SDD reloads both operands per block anyway: one block per wave
 SCHEDULE_SOFTMAX = (4, 4)
+SOFTMAX_LONGEST_FIRST = True     # long rows are dispatched first: they would otherwise finish on a draining machine
 SOFTMAX_WAVES_LONG_ROWS = 8
 ATTENTION_WAVES_LONG_GROUPS = 8
 SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
@@ -112,7 +113,7 @@ def _softmax_schedule(layout, dtype, backward):
         # a row too long for the register-resident walk is streamed by the waves of ONE workgroup (a row
         # cannot be split across workgroups): as many waves as a workgroup holds keep its chunks short
         waves = SOFTMAX_WAVES_LONG_ROWS
-    return schedule_for(layout, (cap, waves, False, slice_max, SOFTMAX_SLICES[which]))
+    return schedule_for(layout, (cap, waves, False, slice_max, SOFTMAX_SLICES[which], SOFTMAX_LONGEST_FIRST))
 
 
 def _check_layout(layout, name):

@@ -140,17 +140,19 @@ def test_schedule_covers_every_pair_once(name, mask, cap, waves, split, longest)
 
 
 @pytest.mark.parametrize("name,mask", _more_masks())
+@pytest.mark.parametrize("longest", [False, True])
 @pytest.mark.parametrize("cap,waves,slice_max,slices", [(4, 4, 24, 2), (4, 4, 3, 4), (2, 2, 0, 2), (4, 8, 64, 4)])
-def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices):
+def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices, longest):
     """Softmax schedules with slice_max: a short row goes whole to `slices` wavefronts (one slice of
     its element rows each) that sit among other sliced rows at the front of the schedule; every
-    other row is chunked as without slicing and never split into parts."""
+    other row is chunked as without slicing and never split into parts.  Longest first, the sliced
+    rows sit by quarters of the longest sliced row's length, and in table order inside a quarter."""
     from sparse import _ops
     mask = np.asarray(mask)
     L = _layout(mask)
     offs = L.row_layout[1].cpu().numpy()
     groups = len(offs) - 1
-    s = _ops.Schedule(L.row_layout[1], L.num_blocks, cap, waves, False, slice_max, slices)
+    s = _ops.Schedule(L.row_layout[1], L.num_blocks, cap, waves, False, slice_max, slices, longest_first=longest)
     raw = s.table.cpu().numpy().reshape(-1, 4)
     meta, tab = raw[:groups], raw[groups: groups + s.workgroups * waves]
     assert (s.tile_slots, s.split_groups) == (0, 0)
@@ -179,6 +181,14 @@ def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices):
         covered[offs[g]: offs[g + 1]] += 1
     assert np.all(covered[: int(offs[-1])] == 1)
     assert last_sliced_wg < first_other_wg                      # sliced rows fill workgroups of their own, first
+    order = [int(g) for slot, (g, b, e, team) in enumerate(tab) if g in slices_seen and ((int(team) >> 8) & 0xFFF) == 0]
+    assert sorted(order) == sorted(sliced)
+    if longest and sliced:
+        yard = max(offs[g + 1] - offs[g] for g in sliced)
+        quarter = lambda n: 0 if 4 * n > 3 * yard else 1 if 2 * n > yard else 2 if 4 * n > yard else 3
+        assert order == sorted(sliced, key=lambda g: (quarter(offs[g + 1] - offs[g]), g))
+    else:
+        assert order == sliced
 
 
 @pytest.mark.parametrize("name,mask", _more_masks())
