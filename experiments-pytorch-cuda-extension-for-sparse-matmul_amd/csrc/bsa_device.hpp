@@ -106,6 +106,21 @@ __device__ __forceinline__ bool map_workgroup(int n_swg, int batches, int &batch
     return batch < batches;
 }
 
+// The same grid for kernels without a dense operand (the softmax reads and writes every byte
+// once, so there is nothing to keep in an L2): schedule order first, i.e. workgroup s of every
+// batch entry is dispatched before workgroup s + 1 of any.  A schedule lists long work first, and
+// in batch-major order the long rows of the last batch entries would start near the end of the
+// launch and finish on an empty machine.
+__device__ __forceinline__ bool map_workgroup_schedule_major(int n_swg, int batches, int &batch, int &swg)
+{
+    int w = (int)blockIdx.x;
+    int t = w >> 3;
+    const int nb8 = (batches + 7) >> 3;
+    batch = (w & 7) + 8 * (t % nb8);
+    swg = t / nb8;
+    return batch < batches;
+}
+
 // Orders the LDS traffic of ONE wavefront: what its lanes wrote before is
 // visible to all its lanes after.  LDS executes a wave's instructions in
 // order, so this only has to stop the compiler from moving accesses across.

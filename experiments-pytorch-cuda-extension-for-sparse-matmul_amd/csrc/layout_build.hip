@@ -134,19 +134,20 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
     const int tid = (int)threadIdx.x;
     int4 *meta = sched;
     int4 *slots = sched + groups;
-    // Serial first-fit in three passes (nine with BSA_SCHED_LONGEST_FIRST).  Row-sliced groups come first and fill whole workgroups of
-    // their own (their waves need no barrier).  Split groups come next: their parts meet in a
-    // workspace after the walk, and workgroups are dispatched in slot order, so starting them first
-    // lets that exchange run while the rest of the launch is still multiplying.  Then the others.
-    // Within the sliced and within the unsplit groups the order is table order, or, longest first, by
-    // length (sliced: quarters of the longest sliced group; unsplit: the longest chunk in quarters of
-    // cap): a wave walks its chunk serially and a launch of these kernels is only one or two rounds of
-    // waves, so a long chunk that starts last (the late rows of a causal mask) runs on an almost empty machine.
+    // Serial first-fit, one pass over the groups per class.  Row-sliced groups fill whole workgroups of
+    // their own (their waves need no barrier).  Split groups come before the unsplit ones: their parts
+    // meet in a workspace after the walk, and workgroups are dispatched in slot order, so starting them
+    // first lets that exchange run while the rest of the launch is still multiplying.
+    // Without BSA_SCHED_LONGEST_FIRST: sliced, split, unsplit, each in table order.  With it, long work
+    // starts first: split groups, then the unsplit ones by their longest chunk (quarters of cap), then the
+    // sliced ones (all shorter than any other group) by length (quarters of the longest of them).  A wave
+    // walks its chunk serially and a launch of these kernels is only one or two rounds of waves, so a long
+    // chunk that starts last (the late rows of a causal mask) runs on an almost empty machine.
     // A team (the waves of one part) never straddles a workgroup boundary.
     if (tid == 0) {
         int pos = 0, tile_slots = 0, split_groups = 0;
         constexpr int LEN_CLASSES = 4;     // by length: > 3/4, > 1/2, > 1/4 of the yardstick, rest
-        const int sliced_passes = longest_first ? LEN_CLASSES : 1;
+        constexpr int CLS_SLICED = 0, CLS_SPLIT = LEN_CLASSES, CLS_UNSPLIT = LEN_CLASSES + 1;
         int longest_sliced = 0;
         if (longest_first)
             for (int g = 0; g < groups; ++g) {
@@ -156,22 +157,28 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
         auto len_class = [](int len, int yard) {
             return 4 * len > 3 * yard ? 0 : (2 * len > yard ? 1 : (4 * len > yard ? 2 : 3));
         };
-        for (int pass = 0; pass < sliced_passes + (longest_first ? 1 + LEN_CLASSES : 2); ++pass) {
+        const int n_pass = longest_first ? 1 + 2 * LEN_CLASSES : 3;
+        for (int pass = 0; pass < n_pass; ++pass) {
+            // class handled by this pass
+            const int want = longest_first ? (pass <= LEN_CLASSES ? CLS_SPLIT + pass : pass - LEN_CLASSES - 1)
+                                           : (pass == 0 ? CLS_SLICED : CLS_SPLIT + pass - 1);
+            // the sliced region starts (and ends) on a workgroup boundary
+            if (want == CLS_SLICED || (!longest_first && want == CLS_SPLIT)) pos = (pos + waves - 1) / waves * waves;
             for (int g = 0; g < groups; ++g) {
                 const GroupPlan gp = plan_group(offsets[g + 1] - offsets[g], cap, waves, allow_split, slice_max, slices);
                 int cls;
                 if (gp.sliced) {
-                    cls = longest_first ? len_class(gp.len, longest_sliced) : 0;
+                    cls = CLS_SLICED + (longest_first ? len_class(gp.len, longest_sliced) : 0);
                 } else if (gp.parts > 1) {
-                    cls = sliced_passes;
+                    cls = CLS_SPLIT;
                 } else {
-                    cls = sliced_passes + 1;
+                    cls = CLS_UNSPLIT;
                     if (longest_first) {
                         const int nw = waves_of_part(gp.len, cap, waves);
                         cls += len_class((gp.len + nw - 1) / nw, cap);   // blocks the busiest wave of the team walks
                     }
                 }
-                if (cls != pass) continue;
+                if (cls != want) continue;
                 if (gp.sliced) {
                     meta[g] = make_int4(pos, -1, -1, gp.parts);
                     pos += gp.parts;
@@ -190,7 +197,6 @@ __global__ __launch_bounds__(LB_THREADS) void schedule_build_kernel(
                 meta[g] = make_int4(first, split ? tile_slots : -1, split ? split_groups : -1, gp.parts);
                 if (split) { tile_slots += gp.parts; split_groups += 1; }
             }
-            if (pass == sliced_passes - 1) pos = (pos + waves - 1) / waves * waves;
         }
         int n_wgs = (pos + waves - 1) / waves;
         total_slots = n_wgs * waves;

@@ -501,7 +501,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
     __shared__ float2 stats[SM_MAX_WAVES][BS];
 
     int batch, swg;
-    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    if (!map_workgroup_schedule_major(n_swg, batches, batch, swg)) return;
     const int w = wave_id(), l = lane_id();
     const int W = (int)(blockDim.x >> 6);
     const SchedEntry e = sched[swg * W + w];
@@ -823,7 +823,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
     __shared__ float dots[SM_MAX_WAVES][BS];
 
     int batch, swg;
-    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    if (!map_workgroup_schedule_major(n_swg, batches, batch, swg)) return;
     const int w = wave_id(), l = lane_id();
     const int W = (int)(blockDim.x >> 6);
     const SchedEntry e = sched[swg * W + w];

@@ -146,7 +146,8 @@ def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices, longest)
     """Softmax schedules with slice_max: a short row goes whole to `slices` wavefronts (one slice of
     its element rows each) that sit among other sliced rows at the front of the schedule; every
     other row is chunked as without slicing and never split into parts.  Longest first, the sliced
-    rows sit by quarters of the longest sliced row's length, and in table order inside a quarter."""
+    rows come behind the others, by quarters of the longest sliced row's length and in table order
+    inside a quarter."""
     from sparse import _ops
     mask = np.asarray(mask)
     L = _layout(mask)
@@ -160,6 +161,7 @@ def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices, longest)
     slices_seen = {g: [] for g in sliced}
     covered = np.zeros(max(int(offs[-1]), 1), dtype=np.int64)
     last_sliced_wg, first_other_wg = -1, s.workgroups
+    first_sliced_wg, last_other_wg = s.workgroups, -1
     for slot, (g, b, e, team) in enumerate(tab):
         if g < 0:
             continue
@@ -170,17 +172,22 @@ def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices, longest)
             assert (b, e) == (offs[g], offs[g + 1]) and nw == 1 and parts == slices and first == in_wg
             slices_seen[g].append((wg, part))
             last_sliced_wg = max(last_sliced_wg, wg)
+            first_sliced_wg = min(first_sliced_wg, wg)
         else:
             assert parts == 1 and part == 0 and first <= in_wg < first + nw <= waves
             covered[b:e] += 1
             first_other_wg = min(first_other_wg, wg)
+            last_other_wg = max(last_other_wg, wg)
             assert meta[g][0] == groups * 0 + (wg * waves + first)
     for g in sliced:
         got = sorted(slices_seen[g])
         assert sorted(p for _, p in got) == list(range(slices)), (g, got)            # every slice once
         covered[offs[g]: offs[g + 1]] += 1
     assert np.all(covered[: int(offs[-1])] == 1)
-    assert last_sliced_wg < first_other_wg                      # sliced rows fill workgroups of their own, first
+    if longest:                                                 # sliced rows fill workgroups of their own: behind the
+        assert last_other_wg < first_sliced_wg                  # longer rows when long work goes first, else in front
+    else:
+        assert last_sliced_wg < first_other_wg
     order = [int(g) for slot, (g, b, e, team) in enumerate(tab) if g in slices_seen and ((int(team) >> 8) & 0xFFF) == 0]
     assert sorted(order) == sorted(sliced)
     if longest and sliced:
