@@ -9,6 +9,11 @@ of Python loops over the blocks, differentiable, and ``to_dense`` fills absent
 blocks with zeros (the reference leaves them uninitialised); other tensors (host
 memory, other dtypes) take a torch gather; a bool mask means the same as the 0/1
 integer mask.
+
+``block=64`` (not in the reference, whose kernels are 32x32x32 only) accepts a mask of
+64x64 blocks: every kept block is run as its 2x2 tiles of 32x32, i.e. the tables, the
+block stack ``[..., 4 * kept, 32, 32]`` and every kernel are those of the mask with each
+cell repeated twice along both axes.  No kernel treats a 64x64 block as a unit.
 """
 from typing import Tuple
 
@@ -35,18 +40,26 @@ class _BlockCopy(torch.autograd.Function):
 
 
 class SparseLayout:
-    def __init__(self, pattern: torch.Tensor, device=None):
+    def __init__(self, pattern: torch.Tensor, device=None, block: int = BLOCK):
+        if block not in (BLOCK, 2 * BLOCK):
+            raise ValueError(f"block must be 32 or 64, got {block}")
         if pattern.dim() != 2:
             raise ValueError("pattern must be a 2-D block mask")
-        rows, cols = pattern.shape
+        per_side = block // BLOCK                       # 32x32 tiles along one side of a block
+        rows, cols = pattern.size(0) * per_side, pattern.size(1) * per_side
         if not (1 <= rows <= 32767 and 1 <= cols <= 65535):
-            raise ValueError("pattern shape must be within [1, 32767] x [1, 65535]")
+            raise ValueError("pattern must span [1, 32767] x [1, 65535] tiles of 32x32")
         if device is None:
             device = pattern.device if pattern.is_cuda else torch.device("cuda", torch.cuda.current_device())
         self.pattern = pattern
+        self.block = block
+        self.tile_shape = (rows, cols)                  # the mask the tables describe, in 32x32 tiles
         self.device = torch.device(device)
 
-        mask = (pattern != 0).to(device=self.device, dtype=torch.uint8).contiguous()
+        mask = (pattern != 0).to(device=self.device, dtype=torch.uint8)
+        if per_side > 1:
+            mask = mask.repeat_interleave(per_side, 0).repeat_interleave(per_side, 1)
+        mask = mask.contiguous()
         cells = rows * cols
         row_blocks = torch.empty(2 * cells, dtype=torch.int32, device=self.device)
         col_blocks = torch.empty(2 * cells, dtype=torch.int32, device=self.device)
@@ -61,7 +74,7 @@ class SparseLayout:
                 col_blocks.data_ptr(), col_offsets.data_ptr(), nnz_dev.data_ptr(),
                 workspace.data_ptr(), _k.current_stream()))
         nnz = int(nnz_dev.item())
-        self.num_blocks = nnz
+        self.num_blocks = nnz                           # stored 32x32 tiles: the length of a block stack
         self._mask = mask
         self._ordinals = workspace          # int32[rows * cols]: block index of every stored cell
         # exact-size tensors: the boundary derives nnz from blocks.size(0) / 2 (sparse_kernels.cc:13)
@@ -82,7 +95,7 @@ class SparseLayout:
         return x.is_cuda and x.device == self.device and x.dtype in _COPY_DTYPES
 
     def _copy_blocks(self, x: torch.Tensor, gather: bool) -> torch.Tensor:
-        rows, cols = self.pattern.shape
+        rows, cols = self.tile_shape
         x = x.contiguous()
         lead = x.shape[:-2] if gather else x.shape[:-3]
         shape = lead + ((self.num_blocks, BLOCK, BLOCK) if gather else (rows * BLOCK, cols * BLOCK))
@@ -105,7 +118,7 @@ class SparseLayout:
 
     def to_sparse(self, x: torch.Tensor) -> torch.Tensor:
         """``[..., R*32, C*32]`` -> ``[..., nnz, 32, 32]`` (layout.py:40-45)."""
-        rows, cols = self.pattern.shape
+        rows, cols = self.tile_shape
         if tuple(x.shape[-2:]) != (rows * BLOCK, cols * BLOCK):
             raise ValueError(f"expected [..., {rows * BLOCK}, {cols * BLOCK}], got {tuple(x.shape)}")
         if self._on_device_path(x):
@@ -116,7 +129,7 @@ class SparseLayout:
 
     def to_dense(self, x: torch.Tensor) -> torch.Tensor:
         """``[..., nnz, 32, 32]`` -> ``[..., R*32, C*32]``, absent blocks zero (layout.py:47-57)."""
-        rows, cols = self.pattern.shape
+        rows, cols = self.tile_shape
         if tuple(x.shape[-3:]) != (self.num_blocks, BLOCK, BLOCK):
             raise ValueError(f"expected [..., {self.num_blocks}, 32, 32], got {tuple(x.shape)}")
         if self._on_device_path(x):

@@ -126,3 +126,14 @@ def test_attention_entry_points_validate(k):
     assert full(head=128) == -3 and "head_dim 64" in k.lib.bsa_last_error().decode()
     assert full(dk=None) == -1 and full(delta=None) == -1
     assert full(col_sched=None) == -1 and full(col_waves=0) == -1
+
+
+def test_layout_block_size_is_checked_before_the_device_is_touched():
+    import torch
+    import sparse
+    with pytest.raises(ValueError, match="32 or 64"):
+        sparse.SparseLayout(torch.ones(2, 2, dtype=torch.long), block=48)
+    with pytest.raises(ValueError, match="2-D"):
+        sparse.SparseLayout(torch.ones(2, dtype=torch.long), block=64)
+    with pytest.raises(ValueError, match="tiles"):
+        sparse.SparseLayout(torch.ones(16384, 1, dtype=torch.long), block=64)     # 32768 tile rows
