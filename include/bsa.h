@@ -20,6 +20,9 @@
  *                          a sparse operand stored [batch, nnz, 32, 32]
  *   offsets  int32[G+1]    first pair of every group: G = mask rows for the
  *                          row layout, mask columns for the column layout
+ * In the ROW layout pair p therefore has idx == p (the pairs are in row-major
+ * order themselves); the softmax and the walks over a row layout rely on it and
+ * address block p of a row without waiting for its pair.
  *
  * Schedule format (new in this build), int32[4] records:
  *   [0, groups)   one per group: (first slot, first partial-tile slot or -1,
