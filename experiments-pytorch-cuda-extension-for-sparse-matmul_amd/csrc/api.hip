@@ -300,9 +300,16 @@ static void fill_attention(bsa::AttentionArgs &p, int dtype, const void *q, cons
     p.bf16 = dtype == BSA_BF16;
 }
 
+size_t bsa_attention_workspace_bytes(int sched_tile_slots, int sched_split_groups, int batches, int head_dim)
+{
+    if (batches < 1 || (head_dim != 64 && head_dim != 128)) return 0;
+    return bsa::attention_workspace_bytes(sched_tile_slots, sched_split_groups, batches, head_dim);
+}
+
 int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out, float *lse,
                           const int32_t *row_blocks, const int32_t *row_offsets,
                           const int32_t *sched, int sched_wgs, int sched_waves,
+                          int sched_tile_slots, int sched_split_groups, void *workspace, size_t workspace_bytes,
                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                           float scale, int causal, void *stream)
 {
@@ -311,11 +318,20 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
                              mask_rows, mask_cols, nnz, batches);
     if (rc) return rc;
     if (!q || !k || !v || !out) return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if (sched_tile_slots < 0 || sched_split_groups < 0 || (sched_tile_slots > 0) != (sched_split_groups > 0))
+        return fail(BSA_ERR_INVALID, "%s: schedule split counts %d, %d are inconsistent", who, sched_tile_slots,
+                    sched_split_groups);
+    const size_t ws_need = bsa_attention_workspace_bytes(sched_tile_slots, sched_split_groups, batches, head_dim);
+    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need))
+        return fail(BSA_ERR_INVALID, "%s: workspace of %zu bytes needed, %zu given", who, ws_need, workspace_bytes);
     bsa::AttentionArgs p;
     fill_attention(p, dtype, q, k, v, row_blocks, sched, mask_rows, sched_wgs, sched_waves, mask_rows, mask_cols, nnz,
                    batches, head_dim, scale, causal);
     p.out = out;
     p.lse = lse;
+    p.tile_slots = sched_tile_slots;
+    p.split_groups = sched_split_groups;
+    p.workspace = workspace;
     return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
 }
 

@@ -42,11 +42,35 @@ __device__ __forceinline__ float at_lane_xor32(float x)
 }
 __device__ __forceinline__ float at_finite_or_zero(float m) { return m == -__builtin_inff() ? 0.f : m; }
 
+// Split rows of the forward walk: a block row longer than one workgroup's share is cut into parts
+// that run in different workgroups.  Every part parks (O^T, max, sum) of its 32 queries in the
+// workspace and bumps the row's counter; the part that arrives last merges the parts in part order
+// (so the result does not depend on arrival order), resets the counter and stores the row.  Parked
+// values and counters are read and written with agent-scope accesses that go to L2, and all parts
+// of a (batch, row) run on one XCD, so no cache write-back is needed; the wait on vmcnt orders the
+// parked values before the counter.
+struct AtSplitWorkspace {
+    int *counters;     // [batches][split_groups], zero between launches
+    float *tiles;      // [batches][tile_slots][at_split_tile_floats(head dim)]
+    int tile_slots, split_groups;
+};
+constexpr int at_split_tile_floats(int hd) { return 32 * hd + 2 * WAVE; }   // O^T, then every lane's max and sum
+static size_t at_split_counter_bytes(int split_groups, int batches)
+{
+    return (((size_t)split_groups * batches * sizeof(int)) + 255) / 256 * 256;
+}
+size_t attention_workspace_bytes(int tile_slots, int split_groups, int batches, int head_dim)
+{
+    if (tile_slots <= 0 || split_groups <= 0) return 0;
+    return at_split_counter_bytes(split_groups, batches) +
+           (size_t)tile_slots * batches * at_split_tile_floats(head_dim) * sizeof(float);
+}
+
 template <int HD, bool BF>
 __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
     half_t *__restrict__ out, float *__restrict__ lse, const BlockDesc *__restrict__ blocks,
-    const SchedEntry *__restrict__ sched,
+    const SchedGroup *__restrict__ sched_groups, const SchedEntry *__restrict__ sched, AtSplitWorkspace ws,
     int n_swg, int batches, int rows_q, int rows_k, float scale2 /* scale * log2(e) */, int causal)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -241,6 +265,45 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
                 for (int i = 0; i < 16; ++i) oacc[t][i] += op[(t * 16 + i) * WAVE + l] * f;
         }
         m = M;                                   // the sums are relative to the team's reference point now
+    }
+    if (e.parts() > 1) {
+        constexpr int TILE = at_split_tile_floats(HD);
+        const SchedGroup sg = sched_groups[r];
+        float *tile0 = ws.tiles + ((size_t)batch * ws.tile_slots + sg.tile_slot) * TILE;
+        float *mine = tile0 + (size_t)e.part() * TILE;
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                __hip_atomic_store(mine + (t * 16 + i) * WAVE + l, oacc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + 32 * HD + l, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + 32 * HD + WAVE + l, lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        int *counter = ws.counters + (size_t)batch * ws.split_groups + sg.split_index;
+        int old = 0;
+        if (l == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        old = __builtin_amdgcn_readfirstlane(old);
+        const int parts = e.parts();
+        if (old != parts - 1) return;
+        float M = NEG_INF;
+        for (int p = 0; p < parts; ++p)
+            M = fmaxf(M, __hip_atomic_load(tile0 + (size_t)p * TILE + 32 * HD + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        const float MM = at_finite_or_zero(M);
+        lsum = 0.f;
+#pragma unroll
+        for (int t = 0; t < KT; ++t) oacc[t] = f16v{0};
+        for (int p = 0; p < parts; ++p) {
+            const float *src = tile0 + (size_t)p * TILE;
+            const float f = at_exp2(__hip_atomic_load(src + 32 * HD + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - MM);
+            lsum += __hip_atomic_load(src + 32 * HD + WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+#pragma unroll
+            for (int t = 0; t < KT; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    oacc[t][i] += __hip_atomic_load(src + (t * 16 + i) * WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+        }
+        m = M;
+        if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
     // log2 of the row's sum of exponentials of the scaled scores (what the backward pass needs to
@@ -649,8 +712,14 @@ hipError_t launch_attention_backward_dkdv(const AttentionArgs &p, hipStream_t st
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t st)
 {
     dim3 grid(8u * (unsigned)p.sched_wgs * (unsigned)((p.batches + 7) / 8)), block(64 * p.sched_waves);
+    AtSplitWorkspace ws;
+    ws.tile_slots = p.tile_slots;
+    ws.split_groups = p.split_groups;
+    ws.counters = (int *)p.workspace;
+    ws.tiles = (float *)((char *)p.workspace + at_split_counter_bytes(p.split_groups, p.batches));
 #define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (half_t *)p.out, (float *)p.lse, \
-                    (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
+                    (const BlockDesc *)p.blocks, (const SchedGroup *)p.sched, (const SchedEntry *)p.sched + p.groups, ws, \
+                    p.sched_wgs, p.batches, \
                     32 * p.mask_rows, 32 * p.mask_cols, p.scale * 1.4426950408889634f, p.causal ? 1 : 0
     const size_t lds = (size_t)p.sched_waves * at_lds_per_wave(p.head_dim);
     if (p.head_dim == 64) {

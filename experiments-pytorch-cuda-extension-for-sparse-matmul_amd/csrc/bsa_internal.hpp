@@ -72,6 +72,8 @@ struct AttentionArgs {
     const int32_t *sched = nullptr;
     int groups = 0;                 // block rows (block columns for the column walk)
     int sched_wgs = 0, sched_waves = 0;
+    int tile_slots = 0, split_groups = 0;   // forward only: parked tiles / counters one batch entry needs for its split rows
+    void *workspace = nullptr;
     int mask_rows = 0, mask_cols = 0, batches = 0;
     float scale = 1.f;
     bool causal = false;
@@ -79,6 +81,7 @@ struct AttentionArgs {
     int head_dim = 64;      // 64 or 128
 };
 
+size_t attention_workspace_bytes(int tile_slots, int split_groups, int batches, int head_dim);
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t stream);
 hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t stream);
 hipError_t launch_attention_backward_dkdv(const AttentionArgs &p, hipStream_t stream);   // groups = block columns, head dim 64

@@ -21,7 +21,8 @@ SCHEDULE_SOFTMAX = (4, 4)
 SOFTMAX_LONGEST_FIRST = True     # long rows are dispatched first: they would otherwise finish on a draining machine
 SOFTMAX_WAVES_LONG_ROWS = 8
 ATTENTION_WAVES_LONG_GROUPS = 8
-SCHEDULE_ATTENTION = (16, 4)          # fused forward: rows are never split across workgroups
+ATTENTION_SPLIT_ROWS = True       # forward: rows longer than cap * waves are cut into parts across workgroups
+SCHEDULE_ATTENTION = (12, 4)           # forward: rows of more than 48 blocks are split across workgroups
 SCHEDULE_ATTENTION_BACKWARD = (16, 4)
 SCHEDULE_ATTENTION_BACKWARD_COLUMNS = (8, 8)
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
@@ -68,6 +69,18 @@ class Schedule:
             self._workspaces[key] = ws
         return ws, need
 
+    def attention_workspace(self, batches: int, head_dim: int, stream: int):
+        """The same for the split rows of the fused attention forward."""
+        need = _k.lib.bsa_attention_workspace_bytes(self.tile_slots, self.split_groups, batches, head_dim)
+        if need == 0:
+            return None, 0
+        key = ("attention", batches, head_dim, stream)
+        ws = self._workspaces.get(key)
+        if ws is None:
+            ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
+            self._workspaces[key] = ws
+        return ws, need
+
 
 def schedule_for(layout, kind):
     """Schedule of a ``(blocks, offset_table)`` tuple, built on first use and kept
@@ -96,10 +109,13 @@ def _group_walk_schedule(layout):
     return schedule_for(layout, kind)
 
 
-def _attention_schedule(layout, kind):
-    """Schedule of a fused attention walk: a group is never split across workgroups there, so a table
-    with a group longer than the workgroup's share gets the most waves a workgroup holds."""
+def _attention_schedule(layout, kind, split=False):
+    """Schedule of a fused attention walk.  The backward walks never split a group across workgroups,
+    so a table with a group longer than the workgroup's share gets the most waves a workgroup holds;
+    the forward walk (``split``) cuts such a row into parts that meet in a workspace."""
     cap, waves = kind
+    if split:
+        return schedule_for(layout, (cap, waves, True))
     if _longest_group(layout[1]) > cap * waves:
         waves = ATTENTION_WAVES_LONG_GROUPS
     return schedule_for(layout, (cap, waves, False))
@@ -294,13 +310,16 @@ def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=F
     out = torch.empty_like(q)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device) if return_lse else None
     if out.numel() > 0:
-        sched = _attention_schedule(row_layout, SCHEDULE_ATTENTION)
+        sched = _attention_schedule(row_layout, SCHEDULE_ATTENTION, split=ATTENTION_SPLIT_ROWS)
         with torch.cuda.device(q.device):
+            stream = _k.current_stream()
+            ws, ws_bytes = sched.attention_workspace(batches, head, stream)
             _k.check(_k.lib.bsa_attention_forward(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                 lse.data_ptr() if lse is not None else None,
                 row_blocks.data_ptr(), row_table.data_ptr(), sched.table.data_ptr(), sched.workgroups, sched.waves,
-                mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), _k.current_stream()))
+                sched.tile_slots, sched.split_groups, ws.data_ptr() if ws is not None else None, ws_bytes,
+                mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), stream))
     return (out, lse) if return_lse else out
 
 

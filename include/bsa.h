@@ -202,13 +202,18 @@ int bsa_softmax_backward(int dtype, const void *y, const void *dy, void *dx,
  *   out  [batches, 32 * mask_rows, head_dim]; rows without stored (or unmasked) blocks give zeros
  *   lse  optional (may be NULL) float[batches, 32 * mask_rows]: log2 of every row's sum of
  *        2^(scale * log2(e) * score); +inf for a row that sees nothing.  The backward pass needs it.
- *   tables / schedule: those of the ROW layout; the schedule must be built with
- *   allow_split = 0 and slice_max = -1 (a block row stays inside one workgroup).
+ *   tables / schedule: those of the ROW layout, the schedule built with slice_max = -1.  With
+ *   BSA_SCHED_SPLIT a block row longer than cap * waves is cut into parts that run in different
+ *   workgroups and meet in `workspace` (sched_tile_slots, sched_split_groups: counts_out[1], [2] of
+ *   bsa_schedule_build; bsa_attention_workspace_bytes() bytes, zeroed once by the caller: every launch
+ *   leaves it zero again, so launches ordered on one stream may share it; NULL when nothing is split).
  * fp16 and bf16 only, head_dim 64 or 128 (BSA_ERR_UNSUPPORTED otherwise).
  */
+size_t bsa_attention_workspace_bytes(int sched_tile_slots, int sched_split_groups, int batches, int head_dim);
 int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v, void *out, float *lse,
                           const int32_t *row_blocks, const int32_t *row_offsets,
                           const int32_t *sched, int sched_wgs, int sched_waves,
+                          int sched_tile_slots, int sched_split_groups, void *workspace, size_t workspace_bytes,
                           int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                           float scale, int causal, void *stream);
 
@@ -239,8 +244,8 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
  * a walk over the columns that rebuilds them a second time and accumulates
  *   dk_out = ds^T q,  dv_out = p^T dout [batches, 32 * mask_cols, head_dim].
  * Seven launches in the unfused chain (sparse/matmul.py:27-52 three times over, sparse_softmax_op.cu:43-63).
- * Row tables and schedule as for bsa_attention_forward; column tables with a schedule of their own built the
- * same way (allow_split = 0, slice_max = -1) on col_offsets.  fp16 / bf16, head_dim 64 only
+ * Row tables with a schedule built without BSA_SCHED_SPLIT and with slice_max = -1 (a block row stays inside
+ * one workgroup in these walks); column tables with a schedule of their own built the same way on col_offsets.  fp16 / bf16, head_dim 64 only
  * (BSA_ERR_UNSUPPORTED otherwise: use bsa_attention_backward_scores and two bsa_matmul calls).
  */
 int bsa_attention_backward(int dtype, const void *q, const void *k, const void *v, const void *dout,

@@ -106,13 +106,22 @@ def test_other_entry_points_validate(k):
 
 def test_attention_entry_points_validate(k):
     """Argument checks of the fused attention calls; every case returns before a launch."""
-    fwd = lambda dtype=1, head=64, q=P, rows=4, cols=4, nnz=5, batches=1, wgs=4, waves=4: k.lib.bsa_attention_forward(
-        dtype, q, P, P, P, None, P, P, P, wgs, waves, rows, cols, nnz, batches, head, 1.0, 0, None)
+    fwd = lambda dtype=1, head=64, q=P, rows=4, cols=4, nnz=5, batches=1, wgs=4, waves=4, tiles=0, splits=0, ws=None, \
+        ws_bytes=0: k.lib.bsa_attention_forward(
+            dtype, q, P, P, P, None, P, P, P, wgs, waves, tiles, splits, ws, ws_bytes, rows, cols, nnz, batches, head,
+            1.0, 0, None)
     assert fwd(dtype=0) == -3 and "fp16" in k.lib.bsa_last_error().decode()
     assert fwd(head=32) == -3 and "head_dim" in k.lib.bsa_last_error().decode()
     assert fwd(q=None) == -1
     assert fwd(nnz=17) == -1 and "nnz" in k.lib.bsa_last_error().decode()
     assert fwd(rows=0) == -1 and fwd(batches=0) == -1 and fwd(waves=9) == -1
+    # split rows: counters (padded to 256 bytes) + per slot and batch entry 32 x head floats of O^T and 128 of (max, sum)
+    assert k.lib.bsa_attention_workspace_bytes(0, 0, 3, 64) == 0
+    assert k.lib.bsa_attention_workspace_bytes(5, 2, 3, 64) == 256 + 5 * 3 * (32 * 64 + 128) * 4
+    assert k.lib.bsa_attention_workspace_bytes(5, 2, 3, 128) == 256 + 5 * 3 * (32 * 128 + 128) * 4
+    assert fwd(tiles=3, splits=0) == -1 and "inconsistent" in k.lib.bsa_last_error().decode()
+    assert fwd(tiles=5, splits=2) == -1 and "workspace" in k.lib.bsa_last_error().decode()
+    assert fwd(tiles=5, splits=2, ws=P, ws_bytes=100) == -1 and "workspace" in k.lib.bsa_last_error().decode()
 
     scores = lambda p=P, ds=P, dq=P, head=64, lse=P: k.lib.bsa_attention_backward_scores(
         1, P, P, P, P, P, lse, p, ds, dq, P, P, P, 4, 4, 4, 4, 5, 1, head, 1.0, 0, None)

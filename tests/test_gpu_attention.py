@@ -60,6 +60,48 @@ def test_long_rows_and_multi_dim_batch():
     assert rel_err(out, ref) <= TOL
 
 
+@pytest.mark.parametrize("dtype,head", [(torch.float16, 64), (torch.bfloat16, 64), (torch.float16, 128)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_rows_split_across_workgroups(dtype, head, causal):
+    """Rows longer than one workgroup's share (cap x waves blocks) are cut into parts that meet in a
+    workspace: same result as the oracle and, within rounding, as the unsplit walk; a second launch on
+    the same workspace gives the same bits (the counters are left at zero); with the causal mask whole
+    parts of a row are hidden (their maximum is -inf) and the row statistics still come out right."""
+    import sparse
+    from sparse import _ops
+    rng = np.random.RandomState(9)
+    mask = (rng.rand(6, 200) < 0.03).astype(np.int64)
+    mask[1, :] = 1                      # 200 blocks: four parts
+    mask[3, 10:140] = 1                 # 130 blocks: three parts
+    mask[4, :65] = 1                    # 65 blocks: two parts
+    mask[5, 150:] = 1                   # all right of the diagonal under the causal mask
+    g = torch.Generator().manual_seed(12)
+    mk = lambda n: torch.randn(3, 32 * n, head, generator=g).to(dtype)
+    q, k, v = mk(6), mk(200), mk(200)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    rl, cl = L.row_layout, L.col_layout
+    sched = _ops._attention_schedule(rl, _ops.SCHEDULE_ATTENTION, split=True)
+    assert sched.split_groups >= 3 and sched.tile_slots >= 9
+    run = lambda: _ops.sparse_attention_forward(q.cuda(), k.cuda(), v.cuda(), rl[0], rl[1], 0.11, causal, cl, return_lse=True)
+    out, lse = run()
+    out2, lse2 = run()
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+    tol = TOL if dtype == torch.float16 else 1.6e-2
+    ref = ao.forward(to_np(q), to_np(k), to_np(v), mask, 0.11, causal)
+    assert rel_err(to_np(out), ref) <= tol
+    if causal:
+        assert torch.all(out[:, 160:] == 0) and torch.all(torch.isinf(lse[:, 160:]))
+    try:
+        _ops.ATTENTION_SPLIT_ROWS = False
+        whole, lse_whole = run()
+    finally:
+        _ops.ATTENTION_SPLIT_ROWS = True
+    assert rel_err(to_np(out), to_np(whole)) <= tol
+    seen = torch.isfinite(lse_whole)
+    assert torch.equal(seen, torch.isfinite(lse))
+    assert torch.allclose(lse[seen], lse_whole[seen], rtol=0, atol=2e-3)
+
+
 def test_large_logits_stay_finite():
     out, ref = _run(np.asarray(ZOO["known3x3"]), 1.0, False, std=6.0, seed=2)   # logits of +-300
     assert np.all(np.isfinite(out)) and rel_err(out, ref) <= TOL
