@@ -335,10 +335,26 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
     return check_launch(bsa::launch_attention_forward(p, (hipStream_t)stream), who);
 }
 
+static int check_split_workspace(const char *who, int tile_slots, int split_groups)
+{
+    if (tile_slots < 0 || split_groups < 0 || (tile_slots > 0) != (split_groups > 0))
+        return fail(BSA_ERR_INVALID, "%s: schedule split counts %d, %d are inconsistent", who, tile_slots, split_groups);
+    return BSA_OK;
+}
+
+size_t bsa_attention_backward_workspace_bytes(int row_tile_slots, int row_split_groups, int col_tile_slots,
+                                              int col_split_groups, int batches, int head_dim)
+{
+    if (batches < 1 || (head_dim != 64 && head_dim != 128)) return 0;
+    return bsa::attention_backward_workspace_bytes(row_tile_slots, row_split_groups, col_tile_slots, col_split_groups,
+                                                   batches, head_dim);
+}
+
 int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const void *v, const void *dout,
                                   const void *out, const float *lse, void *p_out, void *ds_out, void *dq_out,
                                   const int32_t *row_blocks, const int32_t *row_offsets,
                                   const int32_t *sched, int sched_wgs, int sched_waves,
+                                  int sched_tile_slots, int sched_split_groups, void *workspace, size_t workspace_bytes,
                                   int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                                   float scale, int causal, void *stream)
 {
@@ -351,6 +367,12 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
     if ((p_out == nullptr) != (ds_out == nullptr))
         return fail(BSA_ERR_INVALID, "%s: p_out and ds_out go together", who);
     if (!p_out && !dq_out) return fail(BSA_ERR_INVALID, "%s: no output asked for", who);
+    rc = check_split_workspace(who, sched_tile_slots, sched_split_groups);
+    if (rc) return rc;
+    const size_t ws_need = dq_out ? bsa_attention_backward_workspace_bytes(sched_tile_slots, sched_split_groups, 0, 0,
+                                                                           batches, head_dim) : 0;
+    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need))
+        return fail(BSA_ERR_INVALID, "%s: workspace of %zu bytes needed, %zu given", who, ws_need, workspace_bytes);
     bsa::AttentionArgs p;
     fill_attention(p, dtype, q, k, v, row_blocks, sched, mask_rows, sched_wgs, sched_waves, mask_rows, mask_cols, nnz,
                    batches, head_dim, scale, causal);
@@ -360,6 +382,9 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
     p.p_out = p_out;
     p.ds_out = ds_out;
     p.dq_out = dq_out;
+    p.tile_slots = sched_tile_slots;
+    p.split_groups = sched_split_groups;
+    p.workspace = workspace;
     return check_launch(bsa::launch_attention_backward_scores(p, (hipStream_t)stream), who);
 }
 
@@ -368,8 +393,11 @@ int bsa_attention_backward(int dtype, const void *q, const void *k, const void *
                            float *delta_ws,
                            const int32_t *row_blocks, const int32_t *row_offsets,
                            const int32_t *row_sched, int row_sched_wgs, int row_sched_waves,
+                           int row_tile_slots, int row_split_groups,
                            const int32_t *col_blocks, const int32_t *col_offsets,
                            const int32_t *col_sched, int col_sched_wgs, int col_sched_waves,
+                           int col_tile_slots, int col_split_groups,
+                           void *workspace, size_t workspace_bytes,
                            int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                            float scale, int causal, void *stream)
 {
@@ -383,6 +411,15 @@ int bsa_attention_backward(int dtype, const void *q, const void *k, const void *
     if (rc) return rc;
     if (!q || !k || !v || !dout || !out || !lse || !dq_out || !dk_out || !dv_out || !delta_ws)
         return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    rc = check_split_workspace(who, row_tile_slots, row_split_groups);
+    if (rc) return rc;
+    rc = check_split_workspace(who, col_tile_slots, col_split_groups);
+    if (rc) return rc;
+    const size_t row_bytes = bsa_attention_backward_workspace_bytes(row_tile_slots, row_split_groups, 0, 0, batches, head_dim);
+    const size_t ws_need = bsa_attention_backward_workspace_bytes(row_tile_slots, row_split_groups, col_tile_slots,
+                                                                  col_split_groups, batches, head_dim);
+    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need))
+        return fail(BSA_ERR_INVALID, "%s: workspace of %zu bytes needed, %zu given", who, ws_need, workspace_bytes);
     bsa::AttentionArgs p;
     fill_attention(p, dtype, q, k, v, row_blocks, row_sched, mask_rows, row_sched_wgs, row_sched_waves, mask_rows,
                    mask_cols, nnz, batches, head_dim, scale, causal);
@@ -391,6 +428,9 @@ int bsa_attention_backward(int dtype, const void *q, const void *k, const void *
     p.dout = dout;
     p.dq_out = dq_out;
     p.delta = delta_ws;
+    p.tile_slots = row_tile_slots;
+    p.split_groups = row_split_groups;
+    p.workspace = workspace;
     rc = check_launch(bsa::launch_attention_backward_scores(p, (hipStream_t)stream), who);
     if (rc) return rc;
     p.blocks = col_blocks;
@@ -398,6 +438,9 @@ int bsa_attention_backward(int dtype, const void *q, const void *k, const void *
     p.groups = mask_cols;
     p.sched_wgs = col_sched_wgs;
     p.sched_waves = col_sched_waves;
+    p.tile_slots = col_tile_slots;
+    p.split_groups = col_split_groups;
+    p.workspace = workspace ? (char *)workspace + row_bytes : nullptr;
     p.dk_out = dk_out;
     p.dv_out = dv_out;
     return check_launch(bsa::launch_attention_backward_dkdv(p, (hipStream_t)stream), who);

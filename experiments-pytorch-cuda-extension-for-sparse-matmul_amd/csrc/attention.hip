@@ -66,6 +66,55 @@ size_t attention_workspace_bytes(int tile_slots, int split_groups, int batches, 
            (size_t)tile_slots * batches * at_split_tile_floats(head_dim) * sizeof(float);
 }
 
+// The backward walks split a group the same way, but their parts only add up (the row statistics are
+// known): a part parks NT accumulator tiles, bumps the counter, and the last to arrive sums in part order.
+template <int NT>
+__device__ __forceinline__ void at_park(const f16v (&acc)[NT], float *dst)
+{
+    const int l = lane_id();
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            __hip_atomic_store(dst + (t * 16 + i) * WAVE + l, acc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// returns the number of parts that had arrived before this one
+__device__ __forceinline__ int at_arrive(int *counter)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    int old = 0;
+    if (lane_id() == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_amdgcn_readfirstlane(old);
+}
+template <int NT>
+__device__ __forceinline__ void at_sum_parts(f16v (&acc)[NT], const float *first, int stride, int parts)
+{
+    const int l = lane_id();
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f16v{0};
+    for (int p = 0; p < parts; ++p) {
+        const float *src = first + (size_t)p * stride;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                acc[t][i] += __hip_atomic_load(src + (t * 16 + i) * WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+// workspace of the two backward walks: [row counters | row tiles of 32 hd floats | column counters | column
+// tiles of 2 x 32 hd floats (dv^T, dk^T)]
+static size_t at_bwd_region_bytes(int tile_slots, int split_groups, int batches, int tile_floats)
+{
+    if (tile_slots <= 0 || split_groups <= 0) return 0;
+    return at_split_counter_bytes(split_groups, batches) + (size_t)tile_slots * batches * tile_floats * sizeof(float);
+}
+size_t attention_backward_workspace_bytes(int row_tile_slots, int row_split_groups, int col_tile_slots,
+                                          int col_split_groups, int batches, int head_dim)
+{
+    return at_bwd_region_bytes(row_tile_slots, row_split_groups, batches, 32 * head_dim) +
+           at_bwd_region_bytes(col_tile_slots, col_split_groups, batches, 64 * head_dim);
+}
+
 template <int HD, bool BF>
 __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
@@ -349,7 +398,8 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
     const half_t *__restrict__ dout, const half_t *__restrict__ out, const float *__restrict__ lse,
     half_t *__restrict__ p_out, half_t *__restrict__ ds_out, half_t *__restrict__ dq_out,
     float *__restrict__ delta_out,
-    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
+    const SchedEntry *__restrict__ sched, AtSplitWorkspace ws,
     int n_swg, int batches, int rows_q, int rows_k, int nnz, float scale, int causal)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -391,7 +441,8 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
         }
         delta += at_lane_xor32(delta);           // the other half of the head dim sits in lane l ^ 32
         const float row_lse = lse[(size_t)batch * rows_q + BS * r + qq];
-        if (delta_out != nullptr && w == e.first_wave() && h == 0) delta_out[(size_t)batch * rows_q + BS * r + qq] = delta;
+        if (delta_out != nullptr && w == e.first_wave() && e.part() == 0 && h == 0)
+            delta_out[(size_t)batch * rows_q + BS * r + qq] = delta;
 
         struct Frag { uint4 kk[KT][2], vv[KT][2]; };
         DescWindow win;
@@ -491,6 +542,16 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) dqacc[t][i] += op[(t * 16 + i) * WAVE + l];
     }
+    if (e.parts() > 1) {                         // a row cut into parts: they add up in the workspace
+        constexpr int TILE = 32 * HD;
+        const SchedGroup sg = sched_groups[r];
+        float *tile0 = ws.tiles + ((size_t)batch * ws.tile_slots + sg.tile_slot) * TILE;
+        at_park<KT>(dqacc, tile0 + (size_t)e.part() * TILE);
+        int *counter = ws.counters + (size_t)batch * ws.split_groups + sg.split_index;
+        if (at_arrive(counter) != e.parts() - 1) return;
+        at_sum_parts<KT>(dqacc, tile0, TILE, e.parts());
+        if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     half_t *drow = dq_out + ((size_t)batch * rows_q + BS * r + qq) * HD + 4 * h;
 #pragma unroll
     for (int t = 0; t < KT; ++t)
@@ -509,8 +570,14 @@ hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t 
     const size_t lds = (size_t)p.sched_waves * at_bwd_lds_per_wave(p.head_dim);
 #define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (const half_t *)p.dout, \
                     (const half_t *)p.out, (const float *)p.lse, (half_t *)p.p_out, (half_t *)p.ds_out, (half_t *)p.dq_out, (float *)p.delta, \
-                    (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
+                    (const BlockDesc *)p.blocks, (const SchedGroup *)p.sched, (const SchedEntry *)p.sched + p.groups, ws, \
+                    p.sched_wgs, p.batches, \
                     32 * p.mask_rows, 32 * p.mask_cols, p.nnz, p.scale, p.causal ? 1 : 0
+    AtSplitWorkspace ws;
+    ws.tile_slots = p.tile_slots;
+    ws.split_groups = p.split_groups;
+    ws.counters = (int *)p.workspace;
+    ws.tiles = (float *)((char *)p.workspace + at_split_counter_bytes(p.split_groups, p.batches));
     if (p.head_dim == 64) {
         if (p.bf16) attention_bwd_scores_kernel<64, true><<<grid, block, lds, st>>>(BSA_AT_ARGS);
         else attention_bwd_scores_kernel<64, false><<<grid, block, lds, st>>>(BSA_AT_ARGS);
@@ -551,7 +618,8 @@ __global__ __launch_bounds__(512) void attention_bwd_dkdv_kernel(
     const half_t *__restrict__ q, const half_t *__restrict__ k, const half_t *__restrict__ v,
     const half_t *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ delta,
     half_t *__restrict__ dk_out, half_t *__restrict__ dv_out,
-    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
+    const SchedEntry *__restrict__ sched, AtSplitWorkspace ws,
     int n_swg, int batches, int rows_q, int rows_k, float scale, int causal)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -651,7 +719,7 @@ __global__ __launch_bounds__(512) void attention_bwd_dkdv_kernel(
     }
 
     // team merge, one accumulator set at a time (the staging tiles hold exactly one): every wave of a
-    // column but the leader parks its part, the leader adds and stores
+    // column but the leader parks its part, the leader adds
     const int slot0 = e.first_wave(), nw = e.team_waves();
     const bool leader = active && w == slot0;
     float *park = reinterpret_cast<float *>(my_lds);
@@ -675,17 +743,34 @@ __global__ __launch_bounds__(512) void attention_bwd_dkdv_kernel(
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[t][i] += op[(t * 16 + i) * WAVE + l];
             }
-            half_t *drow = (which == 0 ? dv_out : dk_out) + ((size_t)batch * rows_k + BS * c + key) * HD + 4 * h;
-#pragma unroll
-            for (int t = 0; t < KT; ++t)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    h4 o;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) o[j] = narrow_16<BF>(acc[t][4 * g + j]);
-                    *reinterpret_cast<h4 *>(drow + 32 * t + 8 * g) = o;
-                }
         }
+    }
+    if (!leader) return;
+    if (e.parts() > 1) {                         // a column cut into parts: they add up in the workspace
+        constexpr int HALF = 32 * HD, TILE = 2 * HALF;       // dv^T then dk^T
+        const SchedGroup sg = sched_groups[c];
+        float *tile0 = ws.tiles + ((size_t)batch * ws.tile_slots + sg.tile_slot) * TILE;
+        at_park<KT>(dvacc, tile0 + (size_t)e.part() * TILE);
+        at_park<KT>(dkacc, tile0 + (size_t)e.part() * TILE + HALF);
+        int *counter = ws.counters + (size_t)batch * ws.split_groups + sg.split_index;
+        if (at_arrive(counter) != e.parts() - 1) return;
+        at_sum_parts<KT>(dvacc, tile0, TILE, e.parts());
+        at_sum_parts<KT>(dkacc, tile0 + HALF, TILE, e.parts());
+        if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        f16v (&acc)[KT] = which == 0 ? dvacc : dkacc;
+        half_t *drow = (which == 0 ? dv_out : dk_out) + ((size_t)batch * rows_k + BS * c + key) * HD + 4 * h;
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                h4 o;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o[j] = narrow_16<BF>(acc[t][4 * g + j]);
+                *reinterpret_cast<h4 *>(drow + 32 * t + 8 * g) = o;
+            }
     }
 }
 
@@ -695,8 +780,14 @@ hipError_t launch_attention_backward_dkdv(const AttentionArgs &p, hipStream_t st
     const size_t lds = (size_t)p.sched_waves * at_bwd_col_lds_per_wave(64);
 #define BSA_AT_ARGS (const half_t *)p.q, (const half_t *)p.k, (const half_t *)p.v, (const half_t *)p.dout, \
                     (const float *)p.lse, (const float *)p.delta, (half_t *)p.dk_out, (half_t *)p.dv_out, \
-                    (const BlockDesc *)p.blocks, (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, \
+                    (const BlockDesc *)p.blocks, (const SchedGroup *)p.sched, (const SchedEntry *)p.sched + p.groups, ws, \
+                    p.sched_wgs, p.batches, \
                     32 * p.mask_rows, 32 * p.mask_cols, p.scale, p.causal ? 1 : 0
+    AtSplitWorkspace ws;
+    ws.tile_slots = p.tile_slots;
+    ws.split_groups = p.split_groups;
+    ws.counters = (int *)p.workspace;
+    ws.tiles = (float *)((char *)p.workspace + at_split_counter_bytes(p.split_groups, p.batches));
     if (lds > 65536) {
         const void *fn = p.bf16 ? (const void *)attention_bwd_dkdv_kernel<64, true>
                                 : (const void *)attention_bwd_dkdv_kernel<64, false>;

@@ -72,7 +72,7 @@ struct AttentionArgs {
     const int32_t *sched = nullptr;
     int groups = 0;                 // block rows (block columns for the column walk)
     int sched_wgs = 0, sched_waves = 0;
-    int tile_slots = 0, split_groups = 0;   // forward only: parked tiles / counters one batch entry needs for its split rows
+    int tile_slots = 0, split_groups = 0;   // parked tiles / counters one batch entry needs for the split groups of this walk
     void *workspace = nullptr;
     int mask_rows = 0, mask_cols = 0, batches = 0;
     float scale = 1.f;
@@ -82,6 +82,9 @@ struct AttentionArgs {
 };
 
 size_t attention_workspace_bytes(int tile_slots, int split_groups, int batches, int head_dim);
+// row walk region first, then the column walk's; either may be empty
+size_t attention_backward_workspace_bytes(int row_tile_slots, int row_split_groups, int col_tile_slots,
+                                          int col_split_groups, int batches, int head_dim);
 hipError_t launch_attention_forward(const AttentionArgs &p, hipStream_t stream);
 hipError_t launch_attention_backward_scores(const AttentionArgs &p, hipStream_t stream);
 hipError_t launch_attention_backward_dkdv(const AttentionArgs &p, hipStream_t stream);   // groups = block columns, head dim 64

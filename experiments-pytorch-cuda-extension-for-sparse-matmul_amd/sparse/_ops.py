@@ -21,10 +21,10 @@ SCHEDULE_SOFTMAX = (4, 4)
 SOFTMAX_LONGEST_FIRST = True     # long rows are dispatched first: they would otherwise finish on a draining machine
 SOFTMAX_WAVES_LONG_ROWS = 8
 ATTENTION_WAVES_LONG_GROUPS = 8
-ATTENTION_SPLIT_ROWS = True       # forward: rows longer than cap * waves are cut into parts across workgroups
+ATTENTION_SPLIT_ROWS = True       # groups longer than cap * waves are cut into parts across workgroups
 SCHEDULE_ATTENTION = (12, 4)           # forward: rows of more than 48 blocks are split across workgroups
-SCHEDULE_ATTENTION_BACKWARD = (16, 4)
-SCHEDULE_ATTENTION_BACKWARD_COLUMNS = (8, 8)
+SCHEDULE_ATTENTION_BACKWARD = (12, 4)
+SCHEDULE_ATTENTION_BACKWARD_COLUMNS = (12, 2)
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
@@ -72,9 +72,18 @@ class Schedule:
     def attention_workspace(self, batches: int, head_dim: int, stream: int):
         """The same for the split rows of the fused attention forward."""
         need = _k.lib.bsa_attention_workspace_bytes(self.tile_slots, self.split_groups, batches, head_dim)
+        return self._zeroed(("attention", batches, head_dim, stream), need)
+
+    def attention_backward_workspace(self, columns, batches: int, head_dim: int, stream: int):
+        """The same for the backward walks: this schedule walks the rows, ``columns`` (or None) the columns."""
+        ct, cg = (columns.tile_slots, columns.split_groups) if columns is not None else (0, 0)
+        need = _k.lib.bsa_attention_backward_workspace_bytes(self.tile_slots, self.split_groups, ct, cg, batches,
+                                                             head_dim)
+        return self._zeroed(("attention_backward", id(columns), batches, head_dim, stream), need)
+
+    def _zeroed(self, key, need):
         if need == 0:
             return None, 0
-        key = ("attention", batches, head_dim, stream)
         ws = self._workspaces.get(key)
         if ws is None:
             ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
@@ -341,14 +350,17 @@ def sparse_attention_backward_scores(q, k, v, dout, out, lse, row_blocks, row_ta
     ds = torch.empty(shape, dtype=q.dtype, device=q.device)
     dq = torch.empty_like(q) if with_dq else None
     if q.numel() > 0:
-        sched = _attention_schedule(row_layout, SCHEDULE_ATTENTION_BACKWARD)
+        sched = _attention_schedule(row_layout, SCHEDULE_ATTENTION_BACKWARD, split=ATTENTION_SPLIT_ROWS)
         with torch.cuda.device(q.device):
+            stream = _k.current_stream()
+            ws, ws_bytes = sched.attention_backward_workspace(None, batches, head, stream) if with_dq else (None, 0)
             _k.check(_k.lib.bsa_attention_backward_scores(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
                 lse.data_ptr(), p.data_ptr(), ds.data_ptr(), dq.data_ptr() if with_dq else None,
                 row_blocks.data_ptr(), row_table.data_ptr(),
-                sched.table.data_ptr(), sched.workgroups, sched.waves, mask_rows, mask_cols, nnz, batches, head,
-                float(scale), int(bool(causal)), _k.current_stream()))
+                sched.table.data_ptr(), sched.workgroups, sched.waves, sched.tile_slots, sched.split_groups,
+                ws.data_ptr() if ws is not None else None, ws_bytes, mask_rows, mask_cols, nnz, batches, head,
+                float(scale), int(bool(causal)), stream))
     return p, ds, dq
 
 
@@ -372,13 +384,17 @@ def sparse_attention_backward(q, k, v, dout, out, lse, row_blocks, row_table, co
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     if q.numel() > 0:
         delta = torch.empty_like(lse)
-        rs = _attention_schedule(row_layout, SCHEDULE_ATTENTION_BACKWARD)
-        cs = _attention_schedule(col_layout, SCHEDULE_ATTENTION_BACKWARD_COLUMNS)
+        rs = _attention_schedule(row_layout, SCHEDULE_ATTENTION_BACKWARD, split=ATTENTION_SPLIT_ROWS)
+        cs = _attention_schedule(col_layout, SCHEDULE_ATTENTION_BACKWARD_COLUMNS, split=ATTENTION_SPLIT_ROWS)
         with torch.cuda.device(q.device):
+            stream = _k.current_stream()
+            ws, ws_bytes = rs.attention_backward_workspace(cs, batches, head, stream)
             _k.check(_k.lib.bsa_attention_backward(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
                 lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(),
                 row_blocks.data_ptr(), row_table.data_ptr(), rs.table.data_ptr(), rs.workgroups, rs.waves,
+                rs.tile_slots, rs.split_groups,
                 col_blocks.data_ptr(), col_table.data_ptr(), cs.table.data_ptr(), cs.workgroups, cs.waves,
-                mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), _k.current_stream()))
+                cs.tile_slots, cs.split_groups, ws.data_ptr() if ws is not None else None, ws_bytes,
+                mask_rows, mask_cols, nnz, batches, head, float(scale), int(bool(causal)), stream))
     return dq, dk, dv

@@ -39,10 +39,11 @@ SIGNATURES = {
     "bsa_attention_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i, _i]),
     "bsa_attention_forward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, ctypes.c_size_t,
                                    _i, _i, _i, _i, _i, _f, _i, _vp]),
+    "bsa_attention_backward_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i, _i, _i, _i]),
     "bsa_attention_backward_scores": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i,
-                                           _i, _i, _i, _i, _i, _f, _i, _vp]),
-    "bsa_attention_backward": (_i, [_i] + [_vp] * 10 + [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i,
-                                                        _i, _i, _i, _i, _i, _f, _i, _vp]),
+                                           _i, _i, _vp, ctypes.c_size_t, _i, _i, _i, _i, _i, _f, _i, _vp]),
+    "bsa_attention_backward": (_i, [_i] + [_vp] * 10 + [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i,
+                                                        _vp, ctypes.c_size_t, _i, _i, _i, _i, _i, _f, _i, _vp]),
 }
 
 

@@ -228,12 +228,17 @@ int bsa_attention_forward(int dtype, const void *q, const void *k, const void *v
  * sparse_smm_gpu.cu:106-181).  The caller finishes with the two products that walk the columns,
  * dk = ds^T q and dv = p^T dout (bsa_matmul, mode 1, transposed first operand), and with
  * dq = ds k as a third one if it passed dq_out = NULL.
- * Same tables, schedule (allow_split = 0, slice_max = -1) and limits as the forward.
+ * Same tables, schedule and limits as the forward; a schedule with split rows needs, when dq_out is
+ * asked for, bsa_attention_backward_workspace_bytes(sched_tile_slots, sched_split_groups, 0, 0, ...) bytes
+ * of workspace under the same rules (zeroed once, left zero).
  */
+size_t bsa_attention_backward_workspace_bytes(int row_tile_slots, int row_split_groups, int col_tile_slots,
+                                              int col_split_groups, int batches, int head_dim);
 int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const void *v, const void *dout,
                                   const void *out, const float *lse, void *p_out, void *ds_out, void *dq_out,
                                   const int32_t *row_blocks, const int32_t *row_offsets,
                                   const int32_t *sched, int sched_wgs, int sched_waves,
+                                  int sched_tile_slots, int sched_split_groups, void *workspace, size_t workspace_bytes,
                                   int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                                   float scale, int causal, void *stream);
 
@@ -244,17 +249,23 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
  * a walk over the columns that rebuilds them a second time and accumulates
  *   dk_out = ds^T q,  dv_out = p^T dout [batches, 32 * mask_cols, head_dim].
  * Seven launches in the unfused chain (sparse/matmul.py:27-52 three times over, sparse_softmax_op.cu:43-63).
- * Row tables with a schedule built without BSA_SCHED_SPLIT and with slice_max = -1 (a block row stays inside
- * one workgroup in these walks); column tables with a schedule of their own built the same way on col_offsets.  fp16 / bf16, head_dim 64 only
- * (BSA_ERR_UNSUPPORTED otherwise: use bsa_attention_backward_scores and two bsa_matmul calls).
+ * Row tables with a schedule built with slice_max = -1; column tables with a schedule of their own built the
+ * same way on col_offsets.  Either schedule may split long groups (BSA_SCHED_SPLIT): their parts add up in
+ * `workspace`, bsa_attention_backward_workspace_bytes(counts_out[1], [2] of the row schedule, of the column
+ * schedule, ...) bytes, zeroed once by the caller and left zero by every launch; NULL when nothing is split.
+ * fp16 / bf16, head_dim 64 only (BSA_ERR_UNSUPPORTED otherwise: use bsa_attention_backward_scores and two
+ * bsa_matmul calls).
  */
 int bsa_attention_backward(int dtype, const void *q, const void *k, const void *v, const void *dout,
                            const void *out, const float *lse, void *dq_out, void *dk_out, void *dv_out,
                            float *delta_ws,
                            const int32_t *row_blocks, const int32_t *row_offsets,
                            const int32_t *row_sched, int row_sched_wgs, int row_sched_waves,
+                           int row_tile_slots, int row_split_groups,
                            const int32_t *col_blocks, const int32_t *col_offsets,
                            const int32_t *col_sched, int col_sched_wgs, int col_sched_waves,
+                           int col_tile_slots, int col_split_groups,
+                           void *workspace, size_t workspace_bytes,
                            int mask_rows, int mask_cols, int nnz, int batches, int head_dim,
                            float scale, int causal, void *stream);
 

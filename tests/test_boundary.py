@@ -123,18 +123,31 @@ def test_attention_entry_points_validate(k):
     assert fwd(tiles=5, splits=2) == -1 and "workspace" in k.lib.bsa_last_error().decode()
     assert fwd(tiles=5, splits=2, ws=P, ws_bytes=100) == -1 and "workspace" in k.lib.bsa_last_error().decode()
 
-    scores = lambda p=P, ds=P, dq=P, head=64, lse=P: k.lib.bsa_attention_backward_scores(
-        1, P, P, P, P, P, lse, p, ds, dq, P, P, P, 4, 4, 4, 4, 5, 1, head, 1.0, 0, None)
+    scores = lambda p=P, ds=P, dq=P, head=64, lse=P, tiles=0, splits=0, ws=None, ws_bytes=0: \
+        k.lib.bsa_attention_backward_scores(1, P, P, P, P, P, lse, p, ds, dq, P, P, P, 4, 4, tiles, splits, ws, ws_bytes,
+                                            4, 4, 5, 1, head, 1.0, 0, None)
     assert scores(ds=None) == -1 and "go together" in k.lib.bsa_last_error().decode()
     assert scores(p=None, ds=None, dq=None) == -1 and "no output" in k.lib.bsa_last_error().decode()
     assert scores(lse=None) == -1
     assert scores(head=96) == -3
 
-    full = lambda head=64, dk=P, delta=P, col_sched=P, col_waves=4: k.lib.bsa_attention_backward(
-        1, P, P, P, P, P, P, P, dk, P, delta, P, P, P, 4, 4, P, P, col_sched, 4, col_waves, 4, 4, 5, 1, head, 1.0, 0, None)
+    assert scores(tiles=2, splits=0) == -1 and "inconsistent" in k.lib.bsa_last_error().decode()
+    assert scores(tiles=4, splits=2) == -1 and "workspace" in k.lib.bsa_last_error().decode()
+
+    full = lambda head=64, dk=P, delta=P, col_sched=P, col_waves=4, rt=0, rs=0, ct=0, cs=0, ws=None, ws_bytes=0: \
+        k.lib.bsa_attention_backward(1, P, P, P, P, P, P, P, dk, P, delta, P, P, P, 4, 4, rt, rs, P, P, col_sched, 4,
+                                     col_waves, ct, cs, ws, ws_bytes, 4, 4, 5, 1, head, 1.0, 0, None)
     assert full(head=128) == -3 and "head_dim 64" in k.lib.bsa_last_error().decode()
     assert full(dk=None) == -1 and full(delta=None) == -1
     assert full(col_sched=None) == -1 and full(col_waves=0) == -1
+    # rows: counters + 32 x head floats per slot; columns: counters + 2 x 32 x head floats per slot (dv, dk)
+    wsb = k.lib.bsa_attention_backward_workspace_bytes
+    assert wsb(0, 0, 0, 0, 3, 64) == 0
+    assert wsb(4, 2, 0, 0, 3, 64) == 256 + 4 * 3 * 32 * 64 * 4
+    assert wsb(4, 2, 5, 1, 3, 64) == 256 + 4 * 3 * 32 * 64 * 4 + 256 + 5 * 3 * 64 * 64 * 4
+    assert full(rt=1, rs=0) == -1 and full(ct=0, cs=3) == -1
+    assert full(ct=5, cs=1) == -1 and "workspace" in k.lib.bsa_last_error().decode()
+    assert full(ct=5, cs=1, ws=P, ws_bytes=1000) == -1
 
 
 def test_layout_block_size_is_checked_before_the_device_is_touched():

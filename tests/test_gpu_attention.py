@@ -102,6 +102,49 @@ def test_rows_split_across_workgroups(dtype, head, causal):
     assert torch.allclose(lse[seen], lse_whole[seen], rtol=0, atol=2e-3)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_backward_groups_split_across_workgroups(dtype, causal):
+    """Rows and columns longer than one workgroup's share in the two backward walks: parts add up in a
+    workspace.  Gradients against the oracle and against the unsplit walks; two launches in a row give
+    the same bits (counters left at zero); the stored-stack row walk (dq with p and ds) splits as well."""
+    import sparse
+    from sparse import _ops
+    rng = np.random.RandomState(21)
+    mask = (rng.rand(104, 104) < 0.02).astype(np.int64)
+    mask[3, :] = 1                      # a row of 104 blocks
+    mask[70, 10:90] = 1                 # a row of ~80
+    mask[:, 5] = 1                      # a column of 104
+    mask[20:100, 99] = 1                # a column of ~80
+    g = torch.Generator().manual_seed(33)
+    mk = lambda: (0.5 * torch.randn(2, 32 * 104, 64, generator=g)).to(dtype)
+    q, k, v, dout = mk(), mk(), mk(), mk()
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    rl, cl = L.row_layout, L.col_layout
+    rs = _ops._attention_schedule(rl, _ops.SCHEDULE_ATTENTION_BACKWARD, split=True)
+    cs = _ops._attention_schedule(cl, _ops.SCHEDULE_ATTENTION_BACKWARD_COLUMNS, split=True)
+    assert rs.split_groups >= 2 and cs.split_groups >= 2
+    qd, kd, vd, dd = q.cuda(), k.cuda(), v.cuda(), dout.cuda()
+    out, lse = _ops.sparse_attention_forward(qd, kd, vd, rl[0], rl[1], 0.125, causal, cl, return_lse=True)
+    run = lambda: _ops.sparse_attention_backward(qd, kd, vd, dd, out, lse, rl[0], rl[1], cl[0], cl[1], 0.125, causal)
+    grads = run()
+    again = run()
+    assert all(torch.equal(a, b) for a, b in zip(grads, again))
+    ref = ao.backward(to_np(q), to_np(k), to_np(v), to_np(dout), mask, 0.125, causal)
+    tol = 4 * TOL if dtype == torch.float16 else 2e-2    # as in test_two_launch_backward
+    for name, got, want in zip(("dq", "dk", "dv"), grads, ref):
+        assert rel_err(to_np(got), want) <= tol, name
+    p, ds, dq = _ops.sparse_attention_backward_scores(qd, kd, vd, dd, out, lse, rl[0], rl[1], 0.125, causal, cl)
+    assert rel_err(to_np(dq), ref[0]) <= tol
+    try:
+        _ops.ATTENTION_SPLIT_ROWS = False
+        whole = run()
+    finally:
+        _ops.ATTENTION_SPLIT_ROWS = True
+    for name, a, b in zip(("dq", "dk", "dv"), grads, whole):
+        assert rel_err(to_np(a), to_np(b)) <= tol, name
+
+
 def test_large_logits_stay_finite():
     out, ref = _run(np.asarray(ZOO["known3x3"]), 1.0, False, std=6.0, seed=2)   # logits of +-300
     assert np.all(np.isfinite(out)) and rel_err(out, ref) <= TOL
