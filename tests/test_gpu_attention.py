@@ -145,6 +145,29 @@ def test_backward_groups_split_across_workgroups(dtype, causal):
         assert rel_err(to_np(a), to_np(b)) <= tol, name
 
 
+def test_split_rows_at_head_dim_128():
+    """The row walk of the backward pass at head dim 128 (four accumulator tiles parked per part)."""
+    import sparse
+    from sparse import _ops
+    mask = np.zeros((4, 120), dtype=np.int64)
+    mask[0, :] = 1
+    mask[1, ::7] = 1
+    mask[2, 30:110] = 1
+    mask[3, 5] = 1
+    g = torch.Generator().manual_seed(5)
+    mk = lambda n: (0.5 * torch.randn(2, 32 * n, 128, generator=g)).half()
+    q, k, v, dout = mk(4), mk(120), mk(120), mk(4)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    rl, cl = L.row_layout, L.col_layout
+    assert _ops._attention_schedule(rl, _ops.SCHEDULE_ATTENTION_BACKWARD, split=True).split_groups == 2
+    out, lse = _ops.sparse_attention_forward(q.cuda(), k.cuda(), v.cuda(), rl[0], rl[1], 0.09, False, cl, return_lse=True)
+    assert rel_err(to_np(out), ao.forward(to_np(q), to_np(k), to_np(v), mask, 0.09, False)) <= TOL
+    p, ds, dq = _ops.sparse_attention_backward_scores(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), out, lse, rl[0], rl[1],
+                                                      0.09, False, cl)
+    ref_dq = ao.backward(to_np(q), to_np(k), to_np(v), to_np(dout), mask, 0.09, False)[0]
+    assert rel_err(to_np(dq), ref_dq) <= 4 * TOL
+
+
 def test_large_logits_stay_finite():
     out, ref = _run(np.asarray(ZOO["known3x3"]), 1.0, False, std=6.0, seed=2)   # logits of +-300
     assert np.all(np.isfinite(out)) and rel_err(out, ref) <= TOL
