@@ -55,19 +55,13 @@ class Schedule:
         self.waves = waves
         self.cap = cap
         self._workspaces = {}
+        self._spares = {}
 
     def workspace(self, mode: int, batches: int, size_m: int, size_n: int, stream: int):
         """Zeroed scratch for split groups, one per (shape, stream): launches on one stream run in
         order and each leaves the buffer zero again; launches on different streams may overlap."""
         need = _k.lib.bsa_matmul_workspace_bytes(mode, self.tile_slots, self.split_groups, batches, size_m, size_n)
-        if need == 0:
-            return None, 0
-        key = (mode, batches, size_m, size_n, stream)
-        ws = self._workspaces.get(key)
-        if ws is None:
-            ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
-            self._workspaces[key] = ws
-        return ws, need
+        return self._zeroed((mode, batches, size_m, size_n, stream), need)
 
     def attention_workspace(self, batches: int, head_dim: int, stream: int):
         """The same for the split rows of the fused attention forward."""
@@ -82,11 +76,23 @@ class Schedule:
         return self._zeroed(("attention_backward", id(columns), batches, head_dim, stream), need)
 
     def _zeroed(self, key, need):
+        """Workspace of ``need`` zero bytes for ``key`` (its last item is the stream).  A buffer must be
+        zero before its first launch, and under graph capture nothing can be zeroed (a fill recorded
+        there only runs at replay, possibly after another graph has used the buffer): the first eager
+        call for a shape therefore prepares a second buffer, which a capture on another stream takes."""
         if need == 0:
             return None, 0
         ws = self._workspaces.get(key)
         if ws is None:
-            ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
+            spares = self._spares.setdefault(key[:-1], [])
+            if torch.cuda.is_current_stream_capturing():
+                if not spares:
+                    raise RuntimeError("first use of this operator and shape under graph capture: call it once "
+                                       "eagerly before capturing (its workspace must be zeroed first)")
+                ws = spares.pop()
+            else:
+                ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
+                spares.append(torch.zeros(need, dtype=torch.uint8, device=self.table.device))
             self._workspaces[key] = ws
         return ws, need
 

@@ -159,3 +159,24 @@ def test_layout_block_size_is_checked_before_the_device_is_touched():
         sparse.SparseLayout(torch.ones(2, dtype=torch.long), block=64)
     with pytest.raises(ValueError, match="tiles"):
         sparse.SparseLayout(torch.ones(16384, 1, dtype=torch.long), block=64)     # 32768 tile rows
+
+
+def test_workspace_is_never_created_under_graph_capture(monkeypatch):
+    """A split-group workspace must be zero before its first launch and nothing can be zeroed while a
+    graph is being captured: the first use of a shape under capture is refused, a later one on another
+    stream takes the buffer an eager call prepared."""
+    import torch
+    from sparse import _ops
+    sched = object.__new__(_ops.Schedule)
+    sched._workspaces, sched._spares = {}, {}
+    assert sched._zeroed(("attention", 2, 64, 7), 0) == (None, 0)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    with pytest.raises(RuntimeError, match="eagerly"):
+        sched._zeroed(("attention", 2, 64, 7), 1024)
+    spare = torch.zeros(1024, dtype=torch.uint8)
+    sched._spares[("attention", 2, 64)] = [spare]
+    ws, need = sched._zeroed(("attention", 2, 64, 7), 1024)
+    assert ws is spare and need == 1024 and sched._spares[("attention", 2, 64)] == []
+    assert sched._zeroed(("attention", 2, 64, 7), 1024)[0] is spare            # kept for that stream
+    with pytest.raises(RuntimeError, match="eagerly"):
+        sched._zeroed(("attention", 2, 64, 8), 1024)                           # a third stream: nothing prepared

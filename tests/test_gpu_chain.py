@@ -45,3 +45,36 @@ def test_config5_chain_fp16():
     rows = L.sparse_positions[:, 0]
     sums.view(4, 12, 256, 32).index_add_(2, rows, p.float().sum(-1))
     assert torch.allclose(sums, torch.ones_like(sums), atol=5e-3)
+
+
+def test_split_groups_under_graph_capture():
+    """Operators whose long groups meet in a workspace, captured into a HIP graph on another stream than
+    the eager warm-up ran on: the capture takes the buffer the warm-up zeroed for it; every replay, with
+    eager launches in between, gives the eager result.  A first use under capture is refused."""
+    import sparse
+    from sparse import _ops
+    mask = np.zeros((130, 130), dtype=np.int64)
+    mask[np.arange(130), np.arange(130)] = 1
+    mask[:, 7] = 1                      # a column of 130 blocks: DDS splits it
+    mask[9, :] = 1                      # a row of 130 blocks: DSD and the attention walks split it
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    g = torch.Generator().manual_seed(3)
+    q, k, v = ((0.5 * torch.randn(2, 32 * 130, 64, generator=g)).half().cuda() for _ in range(3))
+    w = (0.1 * torch.randn(2, L.num_blocks, 32, 32, generator=g)).half().cuda()
+
+    def run():
+        return (sparse.matmul(v, w, "dds", L, True, False), sparse.matmul(w, v, "dsd", L),
+                sparse.attention(q, k, v, L, 0.125, True))
+    with torch.no_grad():
+        eager = run()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = run()
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            for a, b in zip(captured, eager):
+                assert torch.equal(a, b)
+            again = run()                                   # eager work between the replays
+            for a, b in zip(again, eager):
+                assert torch.equal(a, b)
