@@ -34,8 +34,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--sets", type=int, default=6,
                     help="operand sets to rotate over (1 = the same operands every launch, which the 256 MB "
                          "infinity cache then serves)")
