@@ -103,19 +103,21 @@ int bsa_to_dense(int dtype, const void *sparse, void *dense, const uint8_t *mask
  * Splits every group of a table into chunks of about `cap` pairs, one chunk
  * per wavefront, and packs the wavefronts into workgroups of `waves`
  * wavefronts.  `flags`: with BSA_SCHED_SPLIT a group longer than cap * waves
- * pairs is cut into parts of at most that many pairs (matmul); without it the
- * group gets longer chunks (softmax, attention: their rows cannot be split
- * across workgroups).  With BSA_SCHED_LONGEST_FIRST the groups that are not split
- * are placed by the length of their longest chunk, longest first, instead of in
- * table order (a wavefront walks its chunk serially and a launch is only a round
- * or two of wavefronts, so the long chunks of the late rows of a causal mask would
- * otherwise start last; it pays for the DSD / DDS walks, not for the others).
+ * pairs is cut into parts of at most that many pairs, which run in different
+ * workgroups and meet in a workspace (DSD / DDS, the attention walks); without
+ * it the group gets longer chunks (softmax: a row cannot be split across
+ * workgroups).  With BSA_SCHED_LONGEST_FIRST long work is placed first instead
+ * of in table order: split groups, then the unsplit ones by the length of their
+ * longest chunk (quarters of cap), then the row-sliced ones by length (a
+ * wavefront walks its chunk serially and a launch is only a round or two of
+ * wavefronts, so the long rows at the end of a causal mask would otherwise start
+ * last; it pays for the DSD / DDS walks and the softmax, not for the others).
  * Empty groups get one wavefront with an empty chunk (it writes the zeros).
  * With `slice_max` >= 0 (softmax only, at most 64) a group of at most slice_max
  * pairs is not chunked at all: it goes whole to `slices` wavefronts (2 or 4),
  * each taking 32 / slices of its 32 element rows (team word: waves = 1, part =
- * slice, parts = slices), and these wavefronts fill workgroups of their own at
- * the front of the schedule.  The softmax kernels keep such a slice in registers
+ * slice, parts = slices), and these wavefronts fill workgroups of their own, at
+ * the front of the schedule (behind the other groups with BSA_SCHED_LONGEST_FIRST).  The softmax kernels keep such a slice in registers
  * when slices is 4 and the group has at most 48 (fp16) / 24 (fp32) pairs in the
  * forward and 24 / 12 pairs in the backward kernel; other sliced groups are
  * still computed correctly, by a slower two-pass walk.  Pass slice_max = -1 for the matmul schedules.
