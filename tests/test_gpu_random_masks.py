@@ -75,3 +75,41 @@ def test_softmax_and_attention(name, mask):
     for got, want in zip((q.grad, k.grad, v.grad), ao.backward(qn, kn, vn, to_np(dout), mask, scale, causal)):
         assert torch.isfinite(got).all()
         assert rel_err(to_np(got), want) <= 8e-3
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_groups_around_the_split_boundaries(seed):
+    """Rows or columns of 47 to 150 blocks (a group longer than cap * waves pairs is cut into parts that
+    meet in a workspace: 40 pairs in the DSD / DDS walks, 48 or 24 in the attention walks), with full rows,
+    full columns and empty rows thrown in: the fused attention forward and backward, DSD and DDS."""
+    import sparse
+    from sparse import _ops
+    rng = np.random.RandomState(1000 + seed)
+    rows, cols = int(rng.randint(2, 9)), int(rng.choice([47, 48, 49, 65, 96, 97, 130, 150]))
+    if seed % 2:
+        rows, cols = cols, rows
+    mask = (rng.rand(rows, cols) < rng.choice([0.02, 0.1, 0.4])).astype(np.int64)
+    for _ in range(int(rng.randint(1, 4))):
+        if rng.rand() < 0.5:
+            mask[rng.randint(rows), rng.randint(0, max(cols // 3, 1)):] = 1
+        else:
+            mask[rng.randint(0, max(rows // 3, 1)):, rng.randint(cols)] = 1
+    if rng.rand() < 0.3:
+        mask[rng.randint(rows)] = 0
+    causal, batch = bool(rng.randint(2)), int(rng.randint(1, 4))
+    scale = float(rng.choice([0.125, 0.09, 0.5]))
+    g = torch.Generator().manual_seed(int(rng.randint(1 << 30)))
+    mk = lambda n: (0.7 * torch.randn(batch, 32 * n, 64, generator=g)).half()
+    q, k, v, dout = mk(rows), mk(cols), mk(cols), mk(rows)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    rl, cl = L.row_layout, L.col_layout
+    qd, kd, vd, dd = (t.cuda() for t in (q, k, v, dout))
+    out, lse = _ops.sparse_attention_forward(qd, kd, vd, rl[0], rl[1], scale, causal, cl, return_lse=True)
+    assert rel_err(to_np(out), ao.forward(to_np(q), to_np(k), to_np(v), mask, scale, causal)) <= 2e-3
+    grads = _ops.sparse_attention_backward(qd, kd, vd, dd, out, lse, rl[0], rl[1], cl[0], cl[1], scale, causal)
+    for got, want in zip(grads, ao.backward(to_np(q), to_np(k), to_np(v), to_np(dout), mask, scale, causal)):
+        assert rel_err(to_np(got), want) <= 8e-3
+    p = sparse.softmax(sparse.matmul(qd, kd, "sdd", L, False, True), L, scale, causal)
+    assert rel_err(to_np(sparse.matmul(p, vd, "dsd", L)), mo.matmul(to_np(p), to_np(v), "dsd", mask)) <= 2e-3
+    assert rel_err(to_np(sparse.matmul(dd, p, "dds", L, True, False)),
+                   mo.matmul(to_np(dout), to_np(p), "dds", mask, True, False)) <= 2e-3
