@@ -115,7 +115,7 @@ int64_t bsa_schedule_capacity(int groups, int nnz, int cap, int waves)
     // waves: sum over parts of (len / cap + 1) <= nnz / cap + parts, parts <= nnz / (cap * waves) + groups;
     // first-fit padding wastes less than the waves it pads for
     int64_t slots = 2 * (2 * ((int64_t)nnz / cap) + groups + 1) + 2 * waves;
-    slots += 2 * (int64_t)groups;   // row-sliced groups take up to 4 slots each
+    slots += 6 * (int64_t)groups;   // row-sliced groups take up to 8 slots each
     return slots + groups;   // one record per group in front
 }
 
@@ -126,8 +126,11 @@ int bsa_schedule_build(const int32_t *offsets, int groups, int cap, int waves, i
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: unknown flags %d", flags);
     if (slice_max < -1 || slice_max > 64)
         return fail(BSA_ERR_INVALID, "bsa_schedule_build: slice_max %d outside [-1, 64]", slice_max);
-    if (slice_max >= 0 && slices != 2 && slices != 4)
-        return fail(BSA_ERR_INVALID, "bsa_schedule_build: slices must be 2 or 4, got %d", slices);
+    if (slice_max >= 0 && slices != 2 && slices != 4 && slices != 8)
+        return fail(BSA_ERR_INVALID, "bsa_schedule_build: slices must be 2, 4 or 8, got %d", slices);
+    if (slice_max >= 0 && waves % slices != 0)
+        return fail(BSA_ERR_INVALID, "bsa_schedule_build: %d waves per workgroup do not hold whole groups of %d slices",
+                    waves, slices);
     if (!offsets || !sched || !counts_out) return fail(BSA_ERR_INVALID, "bsa_schedule_build: null pointer argument");
     if (groups < 1 || groups > 65535) return fail(BSA_ERR_INVALID, "bsa_schedule_build: %d groups outside [1, 65535]", groups);
     if (cap < 1) return fail(BSA_ERR_INVALID, "bsa_schedule_build: cap %d < 1", cap);

@@ -276,6 +276,9 @@ constexpr int SM_SUBS = BSA_SM_SUBS;
 #endif
 constexpr int SM_FWD_SLICES = BSA_SM_FWD_SLICES;   // slices the register-resident walks are compiled for
 constexpr int SM_BWD_SLICES = 4;
+// fp32 rows take twice the registers per block: eight slices keep rows of up to 24 blocks resident in the
+// backward walk (two inputs), like four slices do for the 16-bit types
+template <typename T> constexpr int sm_bwd_slices() { return sizeof(T) == 4 ? 8 : SM_BWD_SLICES; }
 
 template <int MASK>
 __device__ __forceinline__ float lane_xor(float x)
@@ -833,7 +836,7 @@ __global__ __launch_bounds__(64 * SM_MAX_WAVES) __attribute__((amdgpu_waves_per_
     const int row0 = l / LPR;
 
     if (active && e.parts() > 1) {   // row-sliced waves sit in workgroups of their own
-        softmax_bwd_sliced<T, CBS, SM_BWD_SLICES>(y + boff, dy + boff, dx + boff, blocks, e, scale);
+        softmax_bwd_sliced<T, CBS, sm_bwd_slices<T>()>(y + boff, dy + boff, dx + boff, blocks, e, scale);
         return;
     }
     if (sched[swg * W].parts() > 1) return;
@@ -997,7 +1000,7 @@ hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t 
             (const bf16_t *)p.x, (const bf16_t *)p.dy, (bf16_t *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     else
-        softmax_bwd_kernel<float, 1, 12><<<grid, block, 0, st>>>(
+        softmax_bwd_kernel<float, 1, 24><<<grid, block, 0, st>>>(
             (const float *)p.x, (const float *)p.dy, (float *)p.out, (const BlockDesc *)p.blocks,
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     return hipGetLastError();

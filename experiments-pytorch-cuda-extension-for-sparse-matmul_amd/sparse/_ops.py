@@ -28,8 +28,8 @@ SCHEDULE_ATTENTION_BACKWARD_COLUMNS = (12, 2)
 # block rows of at most this many blocks are handed whole to SOFTMAX_SLICES wavefronts (8 element rows
 # each), which keep them in registers and need no exchange; per dtype: forward, backward (the
 # backward walk keeps two inputs)
-SOFTMAX_SLICE_MAX = {torch.float16: (48, 24), torch.bfloat16: (48, 24), torch.float32: (24, 12)}
-SOFTMAX_SLICES = (4, 4)              # forward, backward
+SOFTMAX_SLICE_MAX = {torch.float16: (48, 24), torch.bfloat16: (48, 24), torch.float32: (24, 24)}
+SOFTMAX_SLICES = {torch.float16: (4, 4), torch.bfloat16: (4, 4), torch.float32: (4, 8)}      # forward, backward
 
 _DTYPES = {torch.float32: _k.BSA_F32, torch.float16: _k.BSA_F16, torch.bfloat16: _k.BSA_BF16}
 
@@ -139,12 +139,13 @@ def _attention_schedule(layout, kind, split=False):
 def _softmax_schedule(layout, dtype, backward):
     cap, waves = SCHEDULE_SOFTMAX
     which = 1 if backward else 0
-    slice_max = SOFTMAX_SLICE_MAX[dtype][which]
+    slice_max, slices = SOFTMAX_SLICE_MAX[dtype][which], SOFTMAX_SLICES[dtype][which]
     if _longest_group(layout[1]) > slice_max:
         # a row too long for the register-resident walk is streamed by the waves of ONE workgroup (a row
         # cannot be split across workgroups): as many waves as a workgroup holds keep its chunks short
         waves = SOFTMAX_WAVES_LONG_ROWS
-    return schedule_for(layout, (cap, waves, False, slice_max, SOFTMAX_SLICES[which], SOFTMAX_LONGEST_FIRST))
+    waves = max(waves, slices)          # the slices of a row share a workgroup
+    return schedule_for(layout, (cap, waves, False, slice_max, slices, SOFTMAX_LONGEST_FIRST))
 
 
 def _check_layout(layout, name):

@@ -114,13 +114,16 @@ int bsa_to_dense(int dtype, const void *sparse, void *dense, const uint8_t *mask
  * last; it pays for the DSD / DDS walks and the softmax, not for the others).
  * Empty groups get one wavefront with an empty chunk (it writes the zeros).
  * With `slice_max` >= 0 (softmax only, at most 64) a group of at most slice_max
- * pairs is not chunked at all: it goes whole to `slices` wavefronts (2 or 4),
- * each taking 32 / slices of its 32 element rows (team word: waves = 1, part =
- * slice, parts = slices), and these wavefronts fill workgroups of their own, at
- * the front of the schedule (behind the other groups with BSA_SCHED_LONGEST_FIRST).  The softmax kernels keep such a slice in registers
- * when slices is 4 and the group has at most 48 (fp16) / 24 (fp32) pairs in the
- * forward and 24 / 12 pairs in the backward kernel; other sliced groups are
- * still computed correctly, by a slower two-pass walk.  Pass slice_max = -1 for the matmul schedules.
+ * pairs is not chunked at all: it goes whole to `slices` wavefronts (2, 4 or 8;
+ * `waves` must be a multiple), each taking 32 / slices of its 32 element rows
+ * (team word: waves = 1, part = slice, parts = slices), and these wavefronts fill
+ * workgroups of their own, at the front of the schedule (behind the other groups
+ * with BSA_SCHED_LONGEST_FIRST).  The softmax kernels keep such a slice in
+ * registers when the group has at most 48 (fp16 / bf16) or 24 (fp32) pairs and
+ * slices is 4 in the forward kernel, and at most 24 pairs in the backward kernel
+ * with slices 4 (fp16 / bf16) or 8 (fp32); other sliced groups are still computed
+ * correctly, by a slower two-pass walk.  Pass slice_max = -1 for the matmul
+ * schedules.
  * No counterpart in the reference, whose grids are (nnz, B) and
  * (B, M/32, N/32) (sparse/native/sparse_smm_gpu.cu:278-279).
  *   sched        device int32[4 * bsa_schedule_capacity(...)]

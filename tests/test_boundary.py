@@ -91,6 +91,8 @@ def test_other_entry_points_validate(k):
     assert "capacity" in k.lib.bsa_last_error().decode()
     assert k.lib.bsa_schedule_build(P, 4, 4, 4, 0, 8, 3, P, 100, P, None) == -1
     assert "slices" in k.lib.bsa_last_error().decode()
+    assert k.lib.bsa_schedule_build(P, 4, 4, 4, 0, 8, 8, P, 100, P, None) == -1       # 4 waves cannot hold 8 slices
+    assert "whole groups" in k.lib.bsa_last_error().decode()
     assert k.lib.bsa_schedule_build(P, 4, 4, 4, 4, -1, 2, P, 100, P, None) == -1
     assert "flags" in k.lib.bsa_last_error().decode()
     assert k.lib.bsa_softmax_forward(3, P, P, P, P, P, 1, 4, 4, 4, 5, 1, 1.0, 0, None) == -3

@@ -141,7 +141,7 @@ def test_schedule_covers_every_pair_once(name, mask, cap, waves, split, longest)
 
 @pytest.mark.parametrize("name,mask", _more_masks())
 @pytest.mark.parametrize("longest", [False, True])
-@pytest.mark.parametrize("cap,waves,slice_max,slices", [(4, 4, 24, 2), (4, 4, 3, 4), (2, 2, 0, 2), (4, 8, 64, 4)])
+@pytest.mark.parametrize("cap,waves,slice_max,slices", [(4, 4, 24, 2), (4, 4, 3, 4), (2, 2, 0, 2), (4, 8, 64, 4), (4, 8, 24, 8)])
 def test_row_sliced_schedule(name, mask, cap, waves, slice_max, slices, longest):
     """Softmax schedules with slice_max: a short row goes whole to `slices` wavefronts (one slice of
     its element rows each) that sit among other sliced rows at the front of the schedule; every

@@ -149,7 +149,7 @@ def test_backward_every_row_length_up_to_26(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-@pytest.mark.parametrize("slice_max,slices", [(64, 2), (64, 4), (5, 4), (5, 2), (-1, 2)])
+@pytest.mark.parametrize("slice_max,slices", [(64, 2), (64, 4), (64, 8), (5, 4), (5, 2), (5, 8), (-1, 2)])
 def test_schedules_the_resident_walk_does_not_take(monkeypatch, dtype, slice_max, slices):
     """Sliced rows longer than the register capacity, or cut into another number of slices than the
     kernel keeps in registers, go through the two-pass walk and give the same result."""
@@ -157,7 +157,7 @@ def test_schedules_the_resident_walk_does_not_take(monkeypatch, dtype, slice_max
     from sparse import _ops
     from sparse.kernel import sparse_ops
     monkeypatch.setattr(_ops, "SOFTMAX_SLICE_MAX", {torch.float16: (slice_max, slice_max), torch.float32: (slice_max, slice_max)})
-    monkeypatch.setattr(_ops, "SOFTMAX_SLICES", (slices, slices))
+    monkeypatch.setattr(_ops, "SOFTMAX_SLICES", {torch.float16: (slices, slices), torch.float32: (slices, slices)})
     mask = np.asarray(ZOO["long_row_5x40"])
     mask = np.concatenate([mask, _tri(40)[:30]], axis=0)
     y, ref = _fwd(mask, dtype, 0.125, True, batch=(2,), std=2.0, seed=9)
