@@ -51,6 +51,8 @@ def main():
                  "communication, so --gpus N > 1 is not implemented.")
 
     import torch
+    import __graft_entry__
+    __graft_entry__.ensure_built()          # loads what is built; compiles only when nothing is
     import sparse
     import workloads as wl
 
