@@ -321,6 +321,18 @@ def main():
         run_config("config5_fused_attention", lambda: sparse.attention(c5["q"], c5["k"], c5["v"], l5, 0.125, False), 4,
                    flops=f5, nbytes=4 * 8192 * 64 * b5 * 2)
         with torch.no_grad():
+            from sparse.kernel import sparse_ops as ops5
+            rl5, cl5 = l5.row_layout, l5.col_layout
+            out5, lse5 = ops5.sparse_attention_forward(c5["q"], c5["k"], c5["v"], rl5[0], rl5[1], 0.125, False, cl5,
+                                                       return_lse=True)
+            dout5 = torch.randn_like(c5["q"])
+        # the two-launch backward of the fused attention: five block products per stored block
+        run_config("config5_fused_attention_backward",
+                   lambda: ops5.sparse_attention_backward(c5["q"], c5["k"], c5["v"], dout5, out5, lse5, rl5[0], rl5[1],
+                                                          cl5[0], cl5[1], 0.125, False), 4,
+                   flops=2.5 * f5, nbytes=(8 * 8192 * 64) * b5 * 2)
+        del out5, lse5, dout5
+        with torch.no_grad():
             sc5 = sparse.matmul(c5["q"], c5["k"], "sdd", l5, False, True)
             p5 = sparse.softmax(sc5, l5, 0.125, False)
         blk5, dense5 = n5 * 1024 * b5 * 2, 8192 * 64 * b5 * 2
