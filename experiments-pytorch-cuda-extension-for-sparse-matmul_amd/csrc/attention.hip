@@ -24,12 +24,6 @@
 
 namespace bsa {
 
-#ifdef BSA_AT_ABLATE   // debug builds: 1 no softmax math, 2 no S product, 4 no PV product, 8 no staging, 16 loads once
-#define AT_ABLATE(bit) ((BSA_AT_ABLATE) & (bit))
-#else
-#define AT_ABLATE(bit) 0
-#endif
-
 // per wave: K tiles (HD / 32 of 2 KB) + V strips (HD / 64 of 4 KB), reused for the O^T partial of the
 // team merge (HD x 32 floats: the same size), + row stats
 constexpr int at_lds_per_wave(int hd) { return 128 * hd + 512; }
@@ -46,9 +40,8 @@ __device__ __forceinline__ float at_finite_or_zero(float m) { return m == -__bui
 // that run in different workgroups.  Every part parks (O^T, max, sum) of its 32 queries in the
 // workspace and bumps the row's counter; the part that arrives last merges the parts in part order
 // (so the result does not depend on arrival order), resets the counter and stores the row.  Parked
-// values and counters are read and written with agent-scope accesses that go to L2, and all parts
-// of a (batch, row) run on one XCD, so no cache write-back is needed; the wait on vmcnt orders the
-// parked values before the counter.
+// values are published and consumed with park_store / split_publish / split_consume / park_load
+// (bsa_device.hpp: release and acquire at agent scope).
 struct AtSplitWorkspace {
     int *counters;     // [batches][split_groups], zero between launches
     float *tiles;      // [batches][tile_slots][at_split_tile_floats(head dim)]
@@ -76,15 +69,7 @@ __device__ __forceinline__ void at_park(const f16v (&acc)[NT], float *dst)
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-            __hip_atomic_store(dst + (t * 16 + i) * WAVE + l, acc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// returns the number of parts that had arrived before this one
-__device__ __forceinline__ int at_arrive(int *counter)
-{
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    int old = 0;
-    if (lane_id() == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return __builtin_amdgcn_readfirstlane(old);
+            park_store(dst + (t * 16 + i) * WAVE + l, acc[t][i]);
 }
 template <int NT>
 __device__ __forceinline__ void at_sum_parts(f16v (&acc)[NT], const float *first, int stride, int parts)
@@ -98,7 +83,7 @@ __device__ __forceinline__ void at_sum_parts(f16v (&acc)[NT], const float *first
         for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i)
-                acc[t][i] += __hip_atomic_load(src + (t * 16 + i) * WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                acc[t][i] += park_load(src + (t * 16 + i) * WAVE + l);
     }
 }
 // workspace of the two backward walks: [row counters | row tiles of 32 hd floats | column counters | column
@@ -172,7 +157,6 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
 
     // registers -> staging tiles; the registers are free for the next block's loads afterwards
     auto stage = [&](const Frag &f) {
-        if (AT_ABLATE(8)) return;
         wave_lds_fence();
 #pragma unroll
         for (int dt = 0; dt < KT; ++dt) lds_put_kc<false>(tile_k + dt * BS2, f.kk[dt]);
@@ -186,18 +170,7 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         for (int dt = 0; dt < KT; ++dt)
 #pragma unroll
             for (int s = 0; s < 2; ++s)
-                if (!AT_ABLATE(2)) sacc = mfma_16<BF>(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
-        if (AT_ABLATE(1)) {
-            h8 pq[2];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) pq[i >> 3][i & 7] = narrow_16<BF>(sacc[i]);
-#pragma unroll
-            for (int t = 0; t < KT; ++t)
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v + (t / 2) * 2048, 32 * (t % 2), s), pq[s], oacc[t]);
-            return;
-        }
+                sacc = mfma_16<BF>(lds_get_kc(tile_k + dt * BS2, s), qop[2 * dt + s], sacc);
 
         // Row maximum of the scaled scores.  Off the diagonal nothing is masked and the scale is
         // folded into the exponent (one fused multiply-add per score); the diagonal block of a
@@ -253,8 +226,7 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         for (int t = 0; t < KT; ++t)
 #pragma unroll
             for (int s = 0; s < 2; ++s)
-                if (!AT_ABLATE(4)) oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v + (t / 2) * 2048, 32 * (t % 2), s), pop[s], oacc[t]);
-                else oacc[t][s] += widen_16<BF>(pop[s][0]);
+                oacc[t] = mfma_16<BF>(lds_get_strip<false>(tile_v + (t / 2) * 2048, 32 * (t % 2), s), pop[s], oacc[t]);
     };
 
     // One block in flight: its tiles are requested as soon as the previous block's have been copied
@@ -268,7 +240,7 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
             load(seg, fr);
             for (int p = seg; p < seg_end; ++p) {
                 stage(fr);
-                if (p + 1 < seg_end && !AT_ABLATE(16)) load(p + 1, fr);
+                if (p + 1 < seg_end) load(p + 1, fr);
                 step(win.get(p).col());
             }
         }
@@ -324,35 +296,32 @@ __global__ __launch_bounds__(512) void attention_fwd_f16_kernel(
         for (int t = 0; t < KT; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i)
-                __hip_atomic_store(mine + (t * 16 + i) * WAVE + l, oacc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(mine + 32 * HD + l, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(mine + 32 * HD + WAVE + l, lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                park_store(mine + (t * 16 + i) * WAVE + l, oacc[t][i]);
+        park_store(mine + 32 * HD + l, m);
+        park_store(mine + 32 * HD + WAVE + l, lsum);
         int *counter = ws.counters + (size_t)batch * ws.split_groups + sg.split_index;
-        int old = 0;
-        if (l == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        old = __builtin_amdgcn_readfirstlane(old);
         const int parts = e.parts();
-        if (old != parts - 1) return;
+        if (split_publish(counter) != parts - 1) return;
+        split_consume();
         float M = NEG_INF;
         for (int p = 0; p < parts; ++p)
-            M = fmaxf(M, __hip_atomic_load(tile0 + (size_t)p * TILE + 32 * HD + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            M = fmaxf(M, park_load(tile0 + (size_t)p * TILE + 32 * HD + l));
         const float MM = at_finite_or_zero(M);
         lsum = 0.f;
 #pragma unroll
         for (int t = 0; t < KT; ++t) oacc[t] = f16v{0};
         for (int p = 0; p < parts; ++p) {
             const float *src = tile0 + (size_t)p * TILE;
-            const float f = at_exp2(__hip_atomic_load(src + 32 * HD + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - MM);
-            lsum += __hip_atomic_load(src + 32 * HD + WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+            const float f = at_exp2(park_load(src + 32 * HD + l) - MM);
+            lsum += park_load(src + 32 * HD + WAVE + l) * f;
 #pragma unroll
             for (int t = 0; t < KT; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
-                    oacc[t][i] += __hip_atomic_load(src + (t * 16 + i) * WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+                    oacc[t][i] += park_load(src + (t * 16 + i) * WAVE + l) * f;
         }
         m = M;
-        if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        split_reset(counter);
     }
     const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
     // log2 of the row's sum of exponentials of the scaled scores (what the backward pass needs to
@@ -548,9 +517,10 @@ __global__ __launch_bounds__(512) void attention_bwd_scores_kernel(
         float *tile0 = ws.tiles + ((size_t)batch * ws.tile_slots + sg.tile_slot) * TILE;
         at_park<KT>(dqacc, tile0 + (size_t)e.part() * TILE);
         int *counter = ws.counters + (size_t)batch * ws.split_groups + sg.split_index;
-        if (at_arrive(counter) != e.parts() - 1) return;
+        if (split_publish(counter) != e.parts() - 1) return;
+        split_consume();
         at_sum_parts<KT>(dqacc, tile0, TILE, e.parts());
-        if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        split_reset(counter);
     }
     half_t *drow = dq_out + ((size_t)batch * rows_q + BS * r + qq) * HD + 4 * h;
 #pragma unroll
@@ -753,10 +723,11 @@ __global__ __launch_bounds__(512) void attention_bwd_dkdv_kernel(
         at_park<KT>(dvacc, tile0 + (size_t)e.part() * TILE);
         at_park<KT>(dkacc, tile0 + (size_t)e.part() * TILE + HALF);
         int *counter = ws.counters + (size_t)batch * ws.split_groups + sg.split_index;
-        if (at_arrive(counter) != e.parts() - 1) return;
+        if (split_publish(counter) != e.parts() - 1) return;
+        split_consume();
         at_sum_parts<KT>(dvacc, tile0, TILE, e.parts());
         at_sum_parts<KT>(dkacc, tile0 + HALF, TILE, e.parts());
-        if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        split_reset(counter);
     }
 #pragma unroll
     for (int which = 0; which < 2; ++which) {

@@ -131,6 +131,62 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// ---- partial results that workgroups hand to one another through global memory ----------------
+// A part of a split group parks its values (park_store), then all its lanes call split_publish();
+// the part that finds every other part arrived calls split_consume() and reads the parked values
+// (park_load).  Which compute units or L2 slices the parts run on plays no role; what orders the
+// accesses is the gfx942 / gfx950 memory model (LLVM AMDGPU backend, "memory model" code sequences):
+//   * park_store / park_load are agent-scope monotonic atomic accesses: they carry sc1, so a store
+//     writes through to the memory every compute unit of the agent sees and a load does not hit in a
+//     cache that is not coherent at agent scope;
+//   * split_publish waits until every parked value of the wave has been acknowledged
+//     (s_waitcnt vmcnt(0): stores count too) before lane 0 bumps the counter with an agent-scope
+//     read-modify-write, which is what a release at agent scope needs after ATOMIC stores (the L2
+//     write-back of the full fence only concerns plain stores);
+//   * the consumer's loads are issued after the counter value is back (a control dependence on its
+//     return value) and are agent-scope atomics themselves, so nothing stale can be served to them.
+// BSA_SPLIT_MODE 1 puts full release / acquire fences around the counter instead, 2 also moves the
+// parked values with plain accesses; both are equivalent under the model and were measured at twice the
+// launch time of the DDS walk (41 against 21 us at 4096 tokens: buffer_wbl2 / buffer_inv per part).
+#ifndef BSA_SPLIT_MODE
+#define BSA_SPLIT_MODE 0
+#endif
+#if BSA_SPLIT_MODE == 2
+__device__ __forceinline__ void park_store(float *p, float v) { *p = v; }
+__device__ __forceinline__ float park_load(const float *p) { return *p; }
+#else
+__device__ __forceinline__ void park_store(float *p, float v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float park_load(const float *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+#endif
+// returns the number of parts that had arrived before this one (uniform across the wave)
+__device__ __forceinline__ int split_publish(int *counter)
+{
+#if BSA_SPLIT_MODE == 0
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#else
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#endif
+    int old = 0;
+    if (lane_id() == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_amdgcn_readfirstlane(old);
+}
+__device__ __forceinline__ void split_consume()
+{
+#if BSA_SPLIT_MODE != 0
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#endif
+}
+__device__ __forceinline__ void split_reset(int *counter)
+{
+    if (lane_id() == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ds_read_b64_tr_b16: inside every group of 16 lanes, source lane s hands in
 // the address of 4 consecutive halves; result lane i receives, as element e,
 // element (i % 4) of source lane 4 * e + i / 4.  With source lane s pointing at
@@ -156,6 +212,14 @@ __device__ __forceinline__ f16v mfma_16(h8 a, h8 b, f16v c)
 {
     if (BF) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+// 16 x 16 x 32 products: operand lane (g = lane / 16, i = lane % 16) holds index i, k = 8 g .. 8 g + 7;
+// accumulator lane (g, i) holds column i (the second operand's index), rows 4 g + v (the first's).
+template <bool BF>
+__device__ __forceinline__ f4v mfma_16x16(h8 a, h8 b, f4v c)
+{
+    if (BF) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 template <bool BF>
 __device__ __forceinline__ half_t narrow_16(float x)      // fp32 -> the 16-bit storage type, round to nearest even

@@ -18,6 +18,8 @@ extern "C" int bsa_lds_access(const char *name, int permuted, int arg0, int arg1
         else if (!strcmp(name, "put_strip_swapped")) a = put_strip_swapped_addr(lane, arg0);
         else if (!strcmp(name, "get_kc_tr_swapped")) a = get_kc_tr_swapped_addr(lane, arg0, arg1);
         else if (!strcmp(name, "get_strip")) a = get_strip_addr(permuted, lane, arg0 & 1, arg0 >> 1, arg1);
+        else if (!strcmp(name, "put_strip16")) a = put_strip16_addr(lane, arg0);
+        else if (!strcmp(name, "get_strip16")) a = get_strip16_addr(lane, arg0, arg1);
         else if (!strcmp(name, "put_result")) a = put_result_addr(lane, arg0);
         else if (!strcmp(name, "get_linear")) a = get_linear_addr(lane, arg0);
         else return -1;
@@ -26,5 +28,7 @@ extern "C" int bsa_lds_access(const char *name, int permuted, int arg0, int arg1
     return 0;
 }
 
+extern "C" int bsa_col16(int t, int i) { return bsa::col16(t, i); }
+extern "C" int bsa_strip16_half_swapped(int k) { return bsa::strip16_half_swapped(k); }
 extern "C" int bsa_perm16(int i) { return bsa::perm16(i); }
 extern "C" int bsa_invperm16(int i) { return bsa::invperm16(i); }

@@ -111,6 +111,30 @@ BSA_HD constexpr int get_strip_addr(bool permuted, int lane, int step, int half,
     return 2 * (k * 64 + x);
 }
 
+// ---- the same [k][64] strip as the row operand of v_mfma_f32_16x16x32 (16 columns x 32 k per product) ----
+// Lane (g = lane / 16, i = lane % 16) of that operand holds k = 8 g .. 8 g + 7 of ONE column, and the
+// accumulator of lane (g, .) holds rows 4 g + v.  Product t (0..3) of a block takes the columns
+//   col16(t, i) = 8 (i / 4) + 32 (t / 2) + 4 (t % 2) + i % 4,
+// so that accumulators t = 0, 1 of a lane are 8 consecutive columns 8 g .. 8 g + 7 and t = 2, 3 the
+// same 32 further on: two 16-byte stores per lane and output row.  A 32-lane phase of the transposing
+// read holds two 16-lane groups whose rows are 8 apart and swizzle alike, each touching one 8-byte
+// half of 16 pieces; rows 8-15 and 24-31 are therefore stored with the two halves of every piece
+// exchanged (bit 3 of k), which sends the two groups to complementary banks.
+BSA_HD constexpr int col16(int t, int i) { return 8 * (i >> 2) + 32 * (t >> 1) + 4 * (t & 1) + (i & 3); }
+BSA_HD constexpr int strip16_half_swapped(int k) { return (k >> 3) & 1; }
+// registers -> LDS: piece c = lane + 64 q as in put_strip_addr; the caller exchanges the halves of
+// the piece when strip16_half_swapped(row) (the row is 8 q + lane / 8, so that is q & 1)
+BSA_HD constexpr int put_strip16_addr(int lane, int q) { return put_strip_addr(lane, q); }
+// address handed to ds_read_b64_tr_b16 for product t; half = 0 for k .. k + 3, 1 for k + 4 .. k + 7
+BSA_HD constexpr int get_strip16_addr(int lane, int t, int half)
+{
+    int g = lane >> 4, s = lane & 15;
+    int k = 8 * g + 4 * half + (s >> 2);
+    int piece = ((s & 3) + 4 * (t >> 1)) ^ strip_swizzle(k);
+    int hp = (t & 1) ^ strip16_half_swapped(k);
+    return 128 * k + 16 * piece + 8 * hp;
+}
+
 // result tile (SDD): lane (row = lane % 32, h = lane / 32) parks columns 16 h .. 16 h + 15
 BSA_HD constexpr int put_result_addr(int lane, int j) { return 16 * kc_slot(lane & 31, 2 * (lane >> 5) + j); }
 BSA_HD constexpr int get_linear_addr(int lane, int q)

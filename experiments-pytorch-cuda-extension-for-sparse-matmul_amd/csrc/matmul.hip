@@ -27,45 +27,14 @@
 // (v) is fed through perm16 so a lane ends up with 16 consecutive output
 // elements; it is always the operand that runs along the contiguous dimension
 // of the output.  The other operand is indexed by the lane.
+#include <cstdlib>
+
 #include "bsa_device.hpp"
 #include "lds_tiles.hpp"
 #include "bsa_internal.hpp"
 #include "../../include/bsa.h"
 
 namespace bsa {
-
-#ifdef BSA_TRACE
-// Debug builds only: per-wave (start, end, hardware id, work) records for timeline studies.
-__device__ unsigned long long *g_trace = nullptr;
-__device__ __forceinline__ void trace_wave(const unsigned long long (&t)[5], int batch, int group, int nblocks)
-{
-    if (g_trace == nullptr || lane_id() != 0) return;
-    unsigned long long t1 = wall_clock64();
-    unsigned hw = __builtin_amdgcn_s_getreg((4) | (0 << 6) | (31 << 11));
-    unsigned xcc = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (31 << 11));
-    unsigned long long i = atomicAdd(g_trace, 1ull);
-    unsigned long long *r = g_trace + 1 + 8 * i;
-    r[0] = t[0]; r[1] = t1; r[2] = ((unsigned long long)xcc << 32) | hw;
-    r[3] = ((unsigned long long)batch << 40) | ((unsigned long long)group << 16) | (unsigned)nblocks;
-    r[4] = t[1]; r[5] = t[2]; r[6] = t[3]; r[7] = t[4];
-}
-#define BSA_TRACE_MARK(i) { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); trace_t[i] = wall_clock64(); }
-#define BSA_TRACE_MARK_NOWAIT(i) { trace_t[i] = wall_clock64(); }
-__device__ int g_ablate = 0;   // 1: no LDS/MFMA, 2: no dense loads, 4: no sparse loads
-#define BSA_ABLATE(bit) (ablate_bits & (bit))
-#define BSA_TRACE_BEGIN const int ablate_bits = __builtin_amdgcn_readfirstlane(g_ablate); unsigned long long trace_t[5]; trace_t[0] = trace_t[1] = trace_t[2] = trace_t[3] = trace_t[4] = wall_clock64();
-#define BSA_TRACE_END(batch, group, n) trace_wave(trace_t, batch, group, n);
-#else
-#ifdef BSA_ABLATE_BITS
-#define BSA_ABLATE(bit) ((BSA_ABLATE_BITS) & (bit))
-#else
-#define BSA_ABLATE(bit) 0
-#endif
-#define BSA_TRACE_MARK(i)
-#define BSA_TRACE_MARK_NOWAIT(i)
-#define BSA_TRACE_BEGIN
-#define BSA_TRACE_END(batch, group, n)
-#endif
 
 constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + 4 KB), reused for the fp32 partial tile
 #ifndef BSA_GW_DEPTH
@@ -324,10 +293,13 @@ __device__ __forceinline__ size_t gw_out_offset(int g, int y0, int yt, int l, in
 }
 
 // Team reduction through LDS + the leader's check.  Returns true for the wave
-// that has to store.  Every wave of the workgroup must call this once.
-__device__ __forceinline__ bool team_reduce(f16v (&acc)[2], const SchedEntry &e, int w,
-                                            unsigned char *lds_raw)
+// that has to store.  Every wave of the workgroup must call this once.  The
+// accumulators are NT vectors of EV floats per lane (2 x 16 for the 32x32x16
+// products, 8 x 4 for the 16x16x32 ones): 32 floats either way.
+template <class V, int NT, int EV>
+__device__ __forceinline__ bool team_reduce(V (&acc)[NT], const SchedEntry &e, int w, unsigned char *lds_raw)
 {
+    static_assert(NT * EV == 32, "a wave owns a 32 x 64 fp32 tile");
     const int l = lane_id();
     const int slot0 = e.first_wave(), nw = e.team_waves();
     const bool active = e.group >= 0;
@@ -336,18 +308,18 @@ __device__ __forceinline__ bool team_reduce(f16v (&acc)[2], const SchedEntry &e,
     if (active && !leader) {
         wave_lds_fence();
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) mine[(t * 16 + v) * WAVE + l] = acc[t][v];
+            for (int v = 0; v < EV; ++v) mine[(t * EV + v) * WAVE + l] = acc[t][v];
     }
     __syncthreads();
     if (leader) {
         for (int o = 1; o < nw; ++o) {
             const float *other = reinterpret_cast<const float *>(lds_raw + (size_t)(w + o) * GW_LDS_PER_WAVE);
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[t][v] += other[(t * 16 + v) * WAVE + l];
+                for (int v = 0; v < EV; ++v) acc[t][v] += other[(t * EV + v) * WAVE + l];
         }
     }
     return leader;
@@ -356,16 +328,16 @@ __device__ __forceinline__ bool team_reduce(f16v (&acc)[2], const SchedEntry &e,
 // Split groups: every part parks its fp32 partial tile in the workspace and bumps
 // the group's counter; the part that arrives last adds the tiles up in part order
 // (so the sum does not depend on arrival order), resets the counter and returns
-// true: it stores the result.  Tiles and counters are read and written with
-// agent-scope accesses that go to L2, and all parts of a (batch, group) run on one
-// XCD, so no cache write-back is needed; the wait on vmcnt orders tile before counter.
+// true: it stores the result.  Publication follows the release / acquire pattern
+// of split_publish / split_consume (bsa_device.hpp).
 struct SplitWorkspace {
     int *counters;     // [batches][strips][split_groups], zero between launches
     float *tiles;      // [batches][strips][tile_slots][2048]
     int tile_slots, split_groups;
 };
 
-__device__ __forceinline__ bool split_combine(f16v (&acc)[2], const SchedEntry &e, const SchedGroup &sg,
+template <class V, int NT, int EV>
+__device__ __forceinline__ bool split_combine(V (&acc)[NT], const SchedEntry &e, const SchedGroup &sg,
                                               const SplitWorkspace &ws, int batch)
 {
     const int l = lane_id();
@@ -374,29 +346,24 @@ __device__ __forceinline__ bool split_combine(f16v (&acc)[2], const SchedEntry &
     float *tile0 = ws.tiles + (cell * ws.tile_slots + sg.tile_slot) * 2048;
     float *mine = tile0 + (size_t)e.part() * 2048;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-            __hip_atomic_store(mine + (t * 16 + v) * WAVE + l, acc[t][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        for (int v = 0; v < EV; ++v) park_store(mine + (t * EV + v) * WAVE + l, acc[t][v]);
     int *counter = ws.counters + cell * ws.split_groups + sg.split_index;
-    int old = 0;
-    if (l == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __builtin_amdgcn_readfirstlane(old);
-    if (old != parts - 1) return false;
+    if (split_publish(counter) != parts - 1) return false;
+    split_consume();
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+        for (int v = 0; v < EV; ++v) acc[t][v] = 0.f;
     for (int p = 0; p < parts; ++p) {
         const float *src = tile0 + (size_t)p * 2048;
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int v = 0; v < 16; ++v)
-                acc[t][v] += __hip_atomic_load(src + (t * 16 + v) * WAVE + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int v = 0; v < EV; ++v) acc[t][v] += park_load(src + (t * EV + v) * WAVE + l);
     }
-    if (l == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    split_reset(counter);
     return true;
 }
 
@@ -413,14 +380,11 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     int n_swg, int batches, int nnz, int DN, int KT, int XT, int sp_shared, int idx_is_pos)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    BSA_TRACE_BEGIN
     int batch, swg;
     if (!map_workgroup(n_swg, batches, batch, swg)) return;   // whole workgroup leaves together
-    if (BSA_ABLATE(32)) return;
     const int w = wave_id(), l = lane_id();
     const int W = (int)(blockDim.x >> 6);
     const SchedEntry e = sched[swg * W + w];
-    if (BSA_ABLATE(64)) { if (e.group == 12345678) out[0] = (half_t)1; return; }
     const int y0 = 64 * (int)blockIdx.y;
     const int ytiles = FULL ? 2 : ((DN - y0) >= 64 ? 2 : 1);
 
@@ -437,7 +401,6 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     auto load_dense = [&](int p, Frag &f) {
         const BlockDesc d = win.get(p);
         const int kblk = S_KC ? d.col() : d.row();
-        if (BSA_ABLATE(2)) return;
         if (D_KC) {          // stored [DN][KT]: two 32 x 32 tiles, rows KT apart
             const half_t *src = dnb + (size_t)y0 * KT + BS * kblk;
             ldg_tile32(src, KT, f.d0);
@@ -456,7 +419,7 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
         }
     };
     auto load = [&](int p, Frag &f) {
-        if (!BSA_ABLATE(4)) ldg_block32_stream(spb + (size_t)win.get(p).idx * BS2, f.s);
+        ldg_block32_stream(spb + (size_t)win.get(p).idx * BS2, f.s);
         load_dense(p, f);
     };
 
@@ -465,10 +428,6 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
     // DSD: the dense strip feeds the accumulator-register index (perm16), the block the lane index;
     // DDS: the other way round.
     auto compute = [&](const Frag &f) {
-        if (BSA_ABLATE(1)) {
-            acc[0][0] += __uint_as_float(f.s[0].x ^ f.s[1].y ^ f.d0[0].x ^ f.d0[1].y ^ f.d1[0].z ^ f.d1[1].w);
-            return;
-        }
         wave_lds_fence();
         if (S_KC) lds_put_kc<!DSD>(tile_s, f.s);
         else lds_put_ks(tile_s, f.s);
@@ -495,20 +454,18 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
                 if (t < ytiles) acc[t] = DSD ? mfma_16<BF>(dop[s][t], sop[s], acc[t]) : mfma_16<BF>(sop[s], dop[s][t], acc[t]);
     };
 
-    BSA_TRACE_MARK_NOWAIT(1)
     if (e.group >= 0) {
         Frag fr[DEPTH];
         for (int seg = e.begin; seg < e.end; seg += WAVE) {
             const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
             win.fetch(blocks, seg, seg_end);
-            if (BSA_ABLATE(128)) { if (win.idx == 12345678) out[0] = (half_t)1; return; }
             int p = seg;
             if (seg_end - seg >= 2 * DEPTH) {
                 // long enough for a steady state in which every load is unconditional.
                 // In a row-major table pair p names block p, so the first block (from HBM, the longest
                 // wait of the wave) is requested without waiting for the descriptors just asked for.
                 if (idx_is_pos) {
-                    if (!BSA_ABLATE(4)) ldg_block32_stream(spb + (size_t)seg * BS2, fr[0].s);
+                    ldg_block32_stream(spb + (size_t)seg * BS2, fr[0].s);
                     load_dense(seg, fr[0]);
                 } else {
                     load(seg, fr[0]);
@@ -527,7 +484,6 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
                 for (int d = 0; d < DEPTH; ++d)
                     if (seg + d < seg_end) load(seg + d, fr[d]);
             }
-            BSA_TRACE_MARK_NOWAIT(2)
             for (; p < seg_end; p += DEPTH) {                // the last pairs: loads only while pairs are left
 #pragma unroll
                 for (int d = 0; d < DEPTH; ++d) {
@@ -540,11 +496,8 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
         }
     }
 
-    BSA_TRACE_MARK(3)
-    if (BSA_ABLATE(256)) { if (acc[0][0] == 1234.5f) out[0] = (half_t)1; return; }
-    const bool store_it = team_reduce(acc, e, w, lds_raw) &&
-                          (e.parts() <= 1 || split_combine(acc, e, sched_groups[e.group], ws, batch));
-    BSA_TRACE_MARK(4)
+    const bool store_it = team_reduce<f16v, 2, 16>(acc, e, w, lds_raw) &&
+                          (e.parts() <= 1 || split_combine<f16v, 2, 16>(acc, e, sched_groups[e.group], ws, batch));
     if (store_it) {
         half_t *ob = out + (size_t)batch * XT * DN;
 #pragma unroll
@@ -558,7 +511,136 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
             }
         }
     }
-    BSA_TRACE_END(batch, e.group, e.end - e.begin)
+}
+
+// ---------------------------------------------------------------------------
+// DSD over a ROW table with the dense operand stored [KT][DN] (the P V product of attention).
+// The stored block is [x][k]: a lane's 8 halves of a 16 x 16 x 32 product (row x = lane % 16,
+// k = 8 (lane / 16) ..) are 16 contiguous bytes of it, and the 64 lanes of one request cover 16
+// whole rows = 1 KB of whole 128-byte lines.  The block therefore goes from global memory straight
+// into operand registers (no LDS write, no LDS read); only the dense strip passes through LDS
+// (put_strip16_addr / get_strip16_addr).  Accumulators: acc[4 xh + t] = rows 16 xh + lane % 16 of
+// the block row, columns col16(t, 4 g + v).
+// ---------------------------------------------------------------------------
+template <int DEPTH, bool BF>
+__global__ __launch_bounds__(512) void dsd_rows_f16_kernel(
+    const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
+    const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
+    const SchedEntry *__restrict__ sched, SplitWorkspace ws,
+    int n_swg, int batches, int nnz, int DN, int KT, int XT, int sp_shared)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;   // whole workgroup leaves together
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const int y0 = 64 * (int)blockIdx.y;
+    const int g = l >> 4, i = l & 15;
+
+    half_t *tile_d = reinterpret_cast<half_t *>(lds_raw + (size_t)w * GW_LDS_PER_WAVE);
+    const half_t *spb = sp + (sp_shared ? 0 : (size_t)batch * nnz * BS2) + i * BS + 8 * g;
+    const half_t *dnb = dn + (size_t)batch * DN * KT + y0;
+
+    struct Frag { uint4 s[2]; uint4 d[4]; };
+    DescWindow win;
+    auto load_block = [&](int idx, Frag &f) {
+        const half_t *b = spb + (size_t)idx * BS2;
+        f.s[0] = ldg16_stream(b);
+        f.s[1] = ldg16_stream(b + 16 * BS);
+    };
+    auto load_dense = [&](int p, Frag &f) {
+        const half_t *src = dnb + (size_t)(BS * win.get(p).col()) * DN;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int c = l + 64 * q;
+            f.d[q] = ldg16(src + (size_t)(c >> 3) * DN + 8 * (c & 7));
+        }
+    };
+    auto load = [&](int p, Frag &f) {
+        load_block(win.get(p).idx, f);
+        load_dense(p, f);
+    };
+
+    f4v acc[8] = {{0}, {0}, {0}, {0}, {0}, {0}, {0}, {0}};
+    auto compute = [&](const Frag &f) {
+        wave_lds_fence();
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            // rows 8-15 and 24-31 (q odd) are stored with the halves of every piece exchanged
+            const uint4 v = (q & 1) ? make_uint4(f.d[q].z, f.d[q].w, f.d[q].x, f.d[q].y) : f.d[q];
+            *reinterpret_cast<uint4 *>(lds_bytes(tile_d) + put_strip16_addr(l, q)) = v;
+        }
+        wave_lds_fence();
+        h8 dop[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            h4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 0)));
+            h4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 1)));
+            dop[t] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int xh = 0; xh < 2; ++xh)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[4 * xh + t] = mfma_16x16<BF>(dop[t], as_h8(f.s[xh]), acc[4 * xh + t]);
+    };
+
+    if (e.group >= 0) {
+        Frag fr[DEPTH];
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+            int p = seg;
+            if (seg_end - seg >= 2 * DEPTH) {
+                // steady state without a conditional load; pair p of a row table names block p, so the
+                // first block (from HBM, the longest wait of the wave) does not wait for the descriptors
+                load_block(seg, fr[0]);
+                load_dense(seg, fr[0]);
+#pragma unroll
+                for (int d = 1; d < DEPTH; ++d) load(seg + d, fr[d]);
+                for (; p + 2 * DEPTH <= seg_end; p += DEPTH) {
+#pragma unroll
+                    for (int d = 0; d < DEPTH; ++d) {
+                        compute(fr[d]);
+                        load(p + d + DEPTH, fr[d]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int d = 0; d < DEPTH; ++d)
+                    if (seg + d < seg_end) load(seg + d, fr[d]);
+            }
+            for (; p < seg_end; p += DEPTH) {                // the last pairs: loads only while pairs are left
+#pragma unroll
+                for (int d = 0; d < DEPTH; ++d) {
+                    if (p + d < seg_end) {
+                        compute(fr[d]);
+                        if (p + d + DEPTH < seg_end) load(p + d + DEPTH, fr[d]);
+                    }
+                }
+            }
+        }
+    }
+
+    const bool store_it = team_reduce<f4v, 8, 4>(acc, e, w, lds_raw) &&
+                          (e.parts() <= 1 || split_combine<f4v, 8, 4>(acc, e, sched_groups[e.group], ws, batch));
+    if (store_it) {
+        half_t *ob = out + (size_t)batch * XT * DN + y0 + 8 * g;
+#pragma unroll
+        for (int xh = 0; xh < 2; ++xh) {
+            half_t *orow = ob + (size_t)(BS * e.group + 16 * xh + i) * DN;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                h8 o;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    o[v] = narrow_16<BF>(acc[4 * xh + 2 * u][v]);
+                    o[4 + v] = narrow_16<BF>(acc[4 * xh + 2 * u + 1][v]);
+                }
+                stg16(orow + 32 * u, __builtin_bit_cast(uint4, o));
+            }
+        }
+    }
 }
 
 template <bool S_KC, bool D_KC, bool DSD>
@@ -607,8 +689,8 @@ __global__ __launch_bounds__(512) void gw_f32_kernel(
             }
         }
     }
-    if (team_reduce(acc, e, w, lds_raw) &&
-        (e.parts() <= 1 || split_combine(acc, e, sched_groups[e.group], ws, batch))) {
+    if (team_reduce<f16v, 2, 16>(acc, e, w, lds_raw) &&
+        (e.parts() <= 1 || split_combine<f16v, 2, 16>(acc, e, sched_groups[e.group], ws, batch))) {
         float *ob = out + (size_t)batch * XT * DN;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -668,6 +750,13 @@ hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t st)
     return b_kc ? launch_sdd_f32<false, true>(p, st) : launch_sdd_f32<false, false>(p, st);
 }
 
+// measurement switch while both walks exist: BSA_GW_LEGACY=1 keeps the LDS-staged block
+static bool gw_direct_rows()
+{
+    static const bool on = [] { const char *v = getenv("BSA_GW_LEGACY"); return !(v && v[0] == '1'); }();
+    return on;
+}
+
 template <bool S_KC, bool D_KC, bool DSD>
 static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const MatmulArgs &p,
                               int DN, int KT, int XT, hipStream_t st)
@@ -684,6 +773,14 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
                     sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0, \
                     p.row_table ? 1 : 0
     const bool full = DN % 64 == 0;
+    if (S_KC && !D_KC && DSD && full && p.row_table && dtype != BSA_F32 && gw_direct_rows()) {
+#define BSA_DR_ARGS (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks, \
+                    sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0
+        if (dtype == BSA_F16) dsd_rows_f16_kernel<GW_PREFETCH_DEPTH, false><<<grid, block, lds, st>>>(BSA_DR_ARGS);
+        else dsd_rows_f16_kernel<GW_PREFETCH_DEPTH, true><<<grid, block, lds, st>>>(BSA_DR_ARGS);
+#undef BSA_DR_ARGS
+        return hipGetLastError();
+    }
     if (dtype == BSA_F16) {
         if (full) gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false, true><<<grid, block, lds, st>>>(BSA_GW_ARGS);
         else gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, false, false><<<grid, block, lds, st>>>(BSA_GW_ARGS);
@@ -732,17 +829,5 @@ hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream
                 : launch_gw_t<false, false, false>(dtype, p.b, p.a, p, DN, KT, XT, st);
 }
 
-#ifdef BSA_TRACE
-}  // namespace bsa
-extern "C" int bsa_debug_trace(unsigned long long *buf)
-{
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(bsa::g_trace), &buf, sizeof(buf));
-}
-extern "C" int bsa_debug_ablate(int bits)
-{
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(bsa::g_ablate), &bits, sizeof(bits));
-}
-namespace bsa {
-#endif
 
 }  // namespace bsa

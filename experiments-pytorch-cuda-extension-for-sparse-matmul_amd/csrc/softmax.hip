@@ -24,13 +24,6 @@
 
 namespace bsa {
 
-#ifdef BSA_TRACE
-__device__ int g_sm_ablate = 0;   // debug builds: 8 = no stores, 16 = no loads
-#define SM_ABLATE(bit) (g_sm_ablate & (bit))
-#else
-#define SM_ABLATE(bit) 0
-#endif
-
 constexpr int SM_MAX_WAVES = 8;
 constexpr int SM_STREAM_REGS = 16;  // 16-byte registers a batch of the streaming walks (rows too long for registers) may hold
 
@@ -346,7 +339,7 @@ __device__ __forceinline__ void softmax_fwd_sliced_body(const T *__restrict__ xb
     for (int t = 0; t < SUBS; ++t) {
 #pragma unroll
         for (int i = 0; i < NI; ++i)
-            raw[t][i] = SM_ABLATE(16) ? make_uint4(off, i, t, map.col0) : ldg16_stream(xrow + chunk_off(t, i));
+            raw[t][i] = ldg16_stream(xrow + chunk_off(t, i));
         __builtin_amdgcn_sched_barrier(0);   // sub-slice t is requested in full before t + 1: it is needed first
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -386,7 +379,7 @@ __device__ __forceinline__ void softmax_fwd_sliced_body(const T *__restrict__ xb
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const bool mine = i < NI - 1 || i * BPI + map.seg < n;
-            if (mine && !SM_ABLATE(8)) stg16_stream(yrow + chunk_off(t, i), C::scaled(raw[t][i], s));
+            if (mine) stg16_stream(yrow + chunk_off(t, i), C::scaled(raw[t][i], s));
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -1005,14 +998,5 @@ hipError_t launch_softmax_backward(int dtype, const SoftmaxArgs &p, hipStream_t 
             (const SchedEntry *)p.sched + p.groups, p.sched_wgs, p.batches, p.nnz, p.scale);
     return hipGetLastError();
 }
-
-#ifdef BSA_TRACE
-}  // namespace bsa
-extern "C" int bsa_debug_sm_ablate(int bits)
-{
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(bsa::g_sm_ablate), &bits, sizeof(bits));
-}
-namespace bsa {
-#endif
 
 }  // namespace bsa

@@ -98,13 +98,15 @@ KERNEL_ACCESSES = [
     ("get_kc_tr_swapped", 8, [dict(arg0=s, arg1=h) for s in (0, 1) for h in (0, 1)]),
     ("get_strip", 8, [dict(permuted=p, arg0=s + 2 * h, arg1=x0)
                       for p in (False, True) for s in (0, 1) for h in (0, 1) for x0 in (0, 32)]),
+    ("put_strip16", 16, [dict(arg0=q) for q in range(4)]),
+    ("get_strip16", 8, [dict(arg0=t, arg1=h) for t in range(4) for h in (0, 1)]),
     ("put_result", 16, [dict(arg0=j) for j in (0, 1)]),
     ("get_linear", 16, [dict(arg0=q) for q in (0, 1)]),
 ]
 
 
 # how the probe binary (csrc/lds_bank_probe.hip) issues each access
-PROBE_OPS = {"put_kc": "w128", "put_ks": "w128", "put_strip": "w128", "put_strip_swapped": "w128", "put_result": "w128",
+PROBE_OPS = {"put_kc": "w128", "put_ks": "w128", "put_strip": "w128", "put_strip_swapped": "w128", "put_result": "w128", "put_strip16": "w128", "get_strip16": "tr64",
              "get_kc": "b128", "get_linear": "b128", "get_ks": "tr64", "get_strip": "tr64", "get_kc_tr_swapped": "tr64"}
 
 
