@@ -151,6 +151,84 @@ size_t bsa_matmul_workspace_bytes(int mode, int sched_tile_slots, int sched_spli
     return bsa::gw_workspace_bytes(sched_tile_slots, sched_split_groups, batches, mode == BSA_DSD ? N : M);
 }
 
+static int matmul_checked(const char *who, bool static_scratch, int mode, int dtype, const void *a, const void *b, void *c,
+                          const int32_t *blocks, const int32_t *offsets, int groups,
+                          const int32_t *sched, int sched_wgs, int sched_waves,
+                          int sched_tile_slots, int sched_split_groups,
+                          void *workspace, size_t workspace_bytes,
+                          int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
+                          int M, int N, int K, int tr_a, int tr_b, void *stream)
+{
+    if (mode != BSA_SDD && mode != BSA_DSD && mode != BSA_DDS)
+        return fail(BSA_ERR_INVALID, "%s: unknown mode %d", who, mode);
+    if (dtype != BSA_F32 && dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: unsupported dtype %d (fp32 = 0, fp16 = 1, bf16 = 2)", who, dtype);
+    // with nnz == 0 the table and the sparse tensor are empty and may be null
+    const bool a_needed = nnz > 0 || mode != BSA_DSD, b_needed = nnz > 0 || mode != BSA_DDS;
+    const bool c_needed = nnz > 0 || mode != BSA_SDD;
+    if ((!a && a_needed) || (!b && b_needed) || (!c && c_needed) || (!blocks && nnz > 0) || !offsets)
+        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
+    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
+        return fail(BSA_ERR_INVALID, "%s: nnz %d does not fit a %d x %d mask", who, nnz, mask_rows, mask_cols);
+    if (batches < 1) return fail(BSA_ERR_INVALID, "%s: batches %d < 1", who, batches);
+    if (sparse_batches != batches && (sparse_batches != 1 || mode == BSA_SDD))
+        return fail(BSA_ERR_INVALID, "%s: sparse_batches must equal batches (%d), or be 1 for dsd / dds; got %d", who,
+                    batches, sparse_batches);
+    if (M < 1 || N < 1 || K < 1 || M % BSA_BLOCK || N % BSA_BLOCK || K % BSA_BLOCK)
+        return fail(BSA_ERR_INVALID, "%s: M, N, K = %d, %d, %d must be positive multiples of %d", who, M, N, K, BSA_BLOCK);
+    int rc = check_schedule(sched, sched_wgs, sched_waves, batches, who);
+    if (rc) return rc;
+
+    // which table the caller must have passed, and what the sparse matrix spans
+    const bool row_table = mode == BSA_SDD || (mode == BSA_DSD && !tr_a) || (mode == BSA_DDS && tr_b);
+    const int want_groups = row_table ? mask_rows : mask_cols;
+    if (groups != want_groups)
+        return fail(BSA_ERR_INVALID, "%s: table has %d groups, the %s layout of a %d x %d mask has %d", who,
+                    groups, row_table ? "row" : "column", mask_rows, mask_cols, want_groups);
+    const int SR = BSA_BLOCK * mask_rows, SC = BSA_BLOCK * mask_cols;
+    if (mode == BSA_SDD) {
+        if (M != SR || N != SC)
+            return fail(BSA_ERR_INVALID, "%s sdd: op(a) has %d rows and op(b) %d columns, the layout spans %d x %d", who,
+                        M, N, SR, SC);
+    } else if (mode == BSA_DSD) {
+        const int m_want = tr_a ? SC : SR, k_want = tr_a ? SR : SC;
+        if (M != m_want || K != k_want)
+            return fail(BSA_ERR_INVALID, "%s dsd: M, K = %d, %d but op(sparse a) is %d x %d", who, M, K, m_want, k_want);
+    } else {
+        const int k_want = tr_b ? SC : SR, n_want = tr_b ? SR : SC;
+        if (K != k_want || N != n_want)
+            return fail(BSA_ERR_INVALID, "%s dds: K, N = %d, %d but op(sparse b) is %d x %d", who, K, N, k_want, n_want);
+    }
+    const int free_dim = mode == BSA_SDD ? K : (mode == BSA_DSD ? N : M);
+    if ((free_dim + 63) / 64 > 65535)
+        return fail(BSA_ERR_INVALID, "%s: dense dimension %d is too large", who, free_dim);
+
+    if (sched_tile_slots < 0 || sched_split_groups < 0 || (sched_tile_slots > 0) != (sched_split_groups > 0))
+        return fail(BSA_ERR_INVALID, "%s: schedule split counts %d, %d are inconsistent", who,
+                    sched_tile_slots, sched_split_groups);
+    const size_t ws_need = bsa_matmul_workspace_bytes(mode, sched_tile_slots, sched_split_groups, batches, M, N);
+    if (static_scratch) {
+        if (ws_need > (size_t)BSA_STATIC_SCRATCH_BYTES)
+            return fail(BSA_ERR_UNSUPPORTED, "%s: the split groups of this schedule need %zu bytes of scratch, the "
+                        "library's static buffer holds %zu (use bsa_matmul with a workspace of the caller's)", who,
+                        ws_need, (size_t)BSA_STATIC_SCRATCH_BYTES);
+    } else if (ws_need > 0 && (!workspace || workspace_bytes < ws_need)) {
+        return fail(BSA_ERR_INVALID, "%s: workspace of %zu bytes needed, %zu given", who, ws_need, workspace_bytes);
+    }
+
+    bsa::MatmulArgs p{a, b, c, blocks, sched, groups, sched_wgs, sched_waves, sched_tile_slots, sched_split_groups,
+                      workspace, nnz, batches, M, N, K, tr_a != 0, tr_b != 0, sparse_batches != batches};
+    p.row_table = row_table;
+    if (nnz == 0 && mode == BSA_SDD) return BSA_OK;   // nothing to write
+    hipError_t err;
+    if (mode == BSA_SDD) err = bsa::launch_sdd(dtype, p, (hipStream_t)stream);
+    else if (static_scratch) err = bsa::launch_group_walk_static_scratch(dtype, mode == BSA_DSD, p, (hipStream_t)stream);
+    else err = bsa::launch_group_walk(dtype, mode == BSA_DSD, p, (hipStream_t)stream);
+    return check_launch(err, who);
+}
+
 int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
                const int32_t *blocks, const int32_t *offsets, int groups,
                const int32_t *sched, int sched_wgs, int sched_waves,
@@ -159,67 +237,23 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
                int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
                int M, int N, int K, int tr_a, int tr_b, void *stream)
 {
-    if (mode != BSA_SDD && mode != BSA_DSD && mode != BSA_DDS)
-        return fail(BSA_ERR_INVALID, "bsa_matmul: unknown mode %d", mode);
-    if (dtype != BSA_F32 && dtype != BSA_F16 && dtype != BSA_BF16)
-        return fail(BSA_ERR_UNSUPPORTED, "bsa_matmul: unsupported dtype %d (fp32 = 0, fp16 = 1, bf16 = 2)", dtype);
-    // with nnz == 0 the table and the sparse tensor are empty and may be null
-    const bool a_needed = nnz > 0 || mode != BSA_DSD, b_needed = nnz > 0 || mode != BSA_DDS;
-    const bool c_needed = nnz > 0 || mode != BSA_SDD;
-    if ((!a && a_needed) || (!b && b_needed) || (!c && c_needed) || (!blocks && nnz > 0) || !offsets)
-        return fail(BSA_ERR_INVALID, "bsa_matmul: null pointer argument");
-    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
-        return fail(BSA_ERR_INVALID, "bsa_matmul: mask shape %d x %d out of range", mask_rows, mask_cols);
-    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
-        return fail(BSA_ERR_INVALID, "bsa_matmul: nnz %d does not fit a %d x %d mask", nnz, mask_rows, mask_cols);
-    if (batches < 1) return fail(BSA_ERR_INVALID, "bsa_matmul: batches %d < 1", batches);
-    if (sparse_batches != batches && (sparse_batches != 1 || mode == BSA_SDD))
-        return fail(BSA_ERR_INVALID, "bsa_matmul: sparse_batches must equal batches (%d), or be 1 for dsd / dds; got %d",
-                    batches, sparse_batches);
-    if (M < 1 || N < 1 || K < 1 || M % BSA_BLOCK || N % BSA_BLOCK || K % BSA_BLOCK)
-        return fail(BSA_ERR_INVALID, "bsa_matmul: M, N, K = %d, %d, %d must be positive multiples of %d", M, N, K, BSA_BLOCK);
-    int rc = check_schedule(sched, sched_wgs, sched_waves, batches, "bsa_matmul");
-    if (rc) return rc;
-
-    // which table the caller must have passed, and what the sparse matrix spans
-    const bool row_table = mode == BSA_SDD || (mode == BSA_DSD && !tr_a) || (mode == BSA_DDS && tr_b);
-    const int want_groups = row_table ? mask_rows : mask_cols;
-    if (groups != want_groups)
-        return fail(BSA_ERR_INVALID, "bsa_matmul: table has %d groups, the %s layout of a %d x %d mask has %d",
-                    groups, row_table ? "row" : "column", mask_rows, mask_cols, want_groups);
-    const int SR = BSA_BLOCK * mask_rows, SC = BSA_BLOCK * mask_cols;
-    if (mode == BSA_SDD) {
-        if (M != SR || N != SC)
-            return fail(BSA_ERR_INVALID, "bsa_matmul sdd: op(a) has %d rows and op(b) %d columns, the layout spans %d x %d",
-                        M, N, SR, SC);
-    } else if (mode == BSA_DSD) {
-        const int m_want = tr_a ? SC : SR, k_want = tr_a ? SR : SC;
-        if (M != m_want || K != k_want)
-            return fail(BSA_ERR_INVALID, "bsa_matmul dsd: M, K = %d, %d but op(sparse a) is %d x %d", M, K, m_want, k_want);
-    } else {
-        const int k_want = tr_b ? SC : SR, n_want = tr_b ? SR : SC;
-        if (K != k_want || N != n_want)
-            return fail(BSA_ERR_INVALID, "bsa_matmul dds: K, N = %d, %d but op(sparse b) is %d x %d", K, N, k_want, n_want);
-    }
-    const int free_dim = mode == BSA_SDD ? K : (mode == BSA_DSD ? N : M);
-    if ((free_dim + 63) / 64 > 65535)
-        return fail(BSA_ERR_INVALID, "bsa_matmul: dense dimension %d is too large", free_dim);
-
-    if (sched_tile_slots < 0 || sched_split_groups < 0 || (sched_tile_slots > 0) != (sched_split_groups > 0))
-        return fail(BSA_ERR_INVALID, "bsa_matmul: schedule split counts %d, %d are inconsistent",
-                    sched_tile_slots, sched_split_groups);
-    const size_t ws_need = bsa_matmul_workspace_bytes(mode, sched_tile_slots, sched_split_groups, batches, M, N);
-    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need))
-        return fail(BSA_ERR_INVALID, "bsa_matmul: workspace of %zu bytes needed, %zu given", ws_need, workspace_bytes);
-
-    bsa::MatmulArgs p{a, b, c, blocks, sched, groups, sched_wgs, sched_waves, sched_tile_slots, sched_split_groups,
-                      workspace, nnz, batches, M, N, K, tr_a != 0, tr_b != 0, sparse_batches != batches};
-    p.row_table = row_table;
-    if (nnz == 0 && mode == BSA_SDD) return BSA_OK;   // nothing to write
-    hipError_t err = mode == BSA_SDD ? bsa::launch_sdd(dtype, p, (hipStream_t)stream)
-                                     : bsa::launch_group_walk(dtype, mode == BSA_DSD, p, (hipStream_t)stream);
-    return check_launch(err, "bsa_matmul");
+    return matmul_checked("bsa_matmul", false, mode, dtype, a, b, c, blocks, offsets, groups, sched, sched_wgs,
+                          sched_waves, sched_tile_slots, sched_split_groups, workspace, workspace_bytes, mask_rows,
+                          mask_cols, nnz, batches, sparse_batches, M, N, K, tr_a, tr_b, stream);
 }
+
+int bsa_matmul_noalloc(int mode, int dtype, const void *a, const void *b, void *c,
+                       const int32_t *blocks, const int32_t *offsets, int groups,
+                       const int32_t *sched, int sched_wgs, int sched_waves,
+                       int sched_tile_slots, int sched_split_groups,
+                       int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
+                       int M, int N, int K, int tr_a, int tr_b, void *stream)
+{
+    return matmul_checked("bsa_matmul_noalloc", true, mode, dtype, a, b, c, blocks, offsets, groups, sched, sched_wgs,
+                          sched_waves, sched_tile_slots, sched_split_groups, nullptr, 0, mask_rows, mask_cols, nnz,
+                          batches, sparse_batches, M, N, K, tr_a, tr_b, stream);
+}
+
 
 static int check_softmax(const char *who, int dtype, const void *p0, const void *p1, const void *p2,
                          const int32_t *blocks, const int32_t *offsets, const int32_t *sched,

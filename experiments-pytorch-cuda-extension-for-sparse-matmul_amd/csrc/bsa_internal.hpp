@@ -40,6 +40,8 @@ size_t gw_counter_bytes(int split_groups, int batches, int free_dim);
 size_t gw_workspace_bytes(int tile_slots, int split_groups, int batches, int free_dim);
 // group walk shared by DSD (dsd = true) and DDS
 hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream_t stream);
+// the same walk with the split-group workspace in the library's static device buffer (p.workspace is ignored)
+hipError_t launch_group_walk_static_scratch(int dtype, bool dsd, const MatmulArgs &p, hipStream_t stream);
 
 struct SoftmaxArgs {
     const void *x;    // forward: scores; backward: y

@@ -28,6 +28,7 @@
 // elements; it is always the operand that runs along the contiguous dimension
 // of the output.  The other operand is indexed by the lane.
 #include <cstdlib>
+#include <mutex>
 
 #include "bsa_device.hpp"
 #include "lds_tiles.hpp"
@@ -805,6 +806,65 @@ size_t gw_workspace_bytes(int tile_slots, int split_groups, int batches, int fre
 {
     return gw_counter_bytes(split_groups, batches, free_dim) +
            (size_t)tile_slots * batches * ((free_dim + 63) / 64) * 2048 * sizeof(float);
+}
+
+// ---------------------------------------------------------------------------
+// The group walk on the library's own scratch buffer, for callers that cannot allocate.
+// `scratch` is device memory of this code object: every GPU the library runs on holds its own
+// copy, at its own address, until the process ends.  In host code the NAME of the array is not a
+// device address; the address is asked for once per device (hipGetSymbolAddress) and kept.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[BSA_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[MAX_DEVICES] = {nullptr};
+
+hipError_t static_scratch(void **ptr)
+{
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return err;
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return hipSuccess;
+}
+}  // namespace
+
+__global__ void clear_ints_kernel(int *p, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+hipError_t launch_group_walk_static_scratch(int dtype, bool dsd, const MatmulArgs &args, hipStream_t st)
+{
+    MatmulArgs p = args;
+    p.workspace = nullptr;
+    const int free_dim = dsd ? p.N : p.M;
+    const size_t need = p.tile_slots > 0 ? gw_workspace_bytes(p.tile_slots, p.split_groups, p.batches, free_dim) : 0;
+    if (need > (size_t)BSA_STATIC_SCRATCH_BYTES) return hipErrorOutOfMemory;   // the C ABI checks first and says why
+    if (need > 0) {
+        void *base = nullptr;
+        hipError_t err = static_scratch(&base);
+        if (err != hipSuccess) return err;
+        // the counters must start at zero and the buffer keeps what the last call left (an earlier launch
+        // may have failed midway); a kernel clears them, so that the call can sit in a captured graph
+        const size_t ints = gw_counter_bytes(p.split_groups, p.batches, free_dim) / sizeof(int);
+        clear_ints_kernel<<<(unsigned)((ints + 255) / 256), 256, 0, st>>>((int *)base, ints);
+        err = hipGetLastError();
+        if (err != hipSuccess) return err;
+        p.workspace = base;
+    }
+    return launch_group_walk(dtype, dsd, p, st);
 }
 
 hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream_t st)

@@ -32,6 +32,8 @@ SIGNATURES = {
     "bsa_matmul_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i, _i, _i, _i]),
     "bsa_matmul": (_i, [_i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp, ctypes.c_size_t,
                         _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "bsa_matmul_noalloc": (_i, [_i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i,
+                                _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "bsa_softmax_forward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "bsa_softmax_backward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
     "bsa_to_sparse": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),

@@ -174,6 +174,28 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
                int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
                int M, int N, int K, int tr_a, int tr_b, void *stream);
 
+/* ---- block-sparse matmul for callers that cannot allocate -----------------
+ * No counterpart in the reference.  For callers that cannot call hipMalloc or hand over a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  Same operation, arguments, checks and results as bsa_matmul (bit for bit: the
+ * kernels are the same), but the partial tiles and counters of split groups live in a buffer
+ * of BSA_STATIC_SCRATCH_BYTES that is part of the library's device code (one copy per GPU,
+ * held until the process ends), so there is no workspace argument and the call allocates
+ * nothing.  A schedule whose split groups need more than that is refused with
+ * BSA_ERR_UNSUPPORTED (bsa_matmul_workspace_bytes() tells the need).  Every call clears the
+ * counters it uses with a small kernel on `stream` before the walk, so the state a previous
+ * call left behind does not matter.  All calls on one GPU share the buffer: calls that may
+ * overlap in time on one GPU (different streams, different threads) race and must be
+ * serialised by the caller.
+ */
+#define BSA_STATIC_SCRATCH_BYTES (16u << 20)
+int bsa_matmul_noalloc(int mode, int dtype, const void *a, const void *b, void *c,
+                       const int32_t *blocks, const int32_t *offsets, int groups,
+                       const int32_t *sched, int sched_wgs, int sched_waves,
+                       int sched_tile_slots, int sched_split_groups,
+                       int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
+                       int M, int N, int K, int tr_a, int tr_b, void *stream);
+
 /* ---- block-sparse softmax ----------------------------------------------
  * Replaces sparse_softmax_forward / sparse_softmax_backward
  * (sparse_softmax.cu:208-258) and their kernels (:113-205), with two additions:
@@ -253,7 +275,7 @@ int bsa_attention_backward_scores(int dtype, const void *q, const void *k, const
  * (and leaves rowsum(dout o out) in `delta_ws`, float [batches, 32 * mask_rows], caller-provided), and
  * a walk over the columns that rebuilds them a second time and accumulates
  *   dk_out = ds^T q,  dv_out = p^T dout [batches, 32 * mask_cols, head_dim].
- * Seven launches in the unfused chain (sparse/matmul.py:27-52 three times over, sparse_softmax_op.cu:43-63).
+ * Seven launches in the unfused chain (sparse/matmul.py:27-52 three times over, sparse_softmax.cu:165-205,233-258).
  * Row tables with a schedule built with slice_max = -1; column tables with a schedule of their own built the
  * same way on col_offsets.  Either schedule may split long groups (BSA_SCHED_SPLIT): their parts add up in
  * `workspace`, bsa_attention_backward_workspace_bytes(counts_out[1], [2] of the row schedule, of the column
