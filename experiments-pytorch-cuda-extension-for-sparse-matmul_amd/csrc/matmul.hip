@@ -27,7 +27,6 @@
 // (v) is fed through perm16 so a lane ends up with 16 consecutive output
 // elements; it is always the operand that runs along the contiguous dimension
 // of the output.  The other operand is indexed by the lane.
-#include <cstdlib>
 #include <mutex>
 
 #include "bsa_device.hpp"
@@ -522,8 +521,13 @@ __global__ __launch_bounds__(512) void gw_f16_kernel(
 // into operand registers (no LDS write, no LDS read); only the dense strip passes through LDS
 // (put_strip16_addr / get_strip16_addr).  Accumulators: acc[4 xh + t] = rows 16 xh + lane % 16 of
 // the block row, columns col16(t, 4 g + v).
+// Pipeline: blocks come from HBM and are requested two steps ahead (two register sets of 8), strips
+// come out of L2 and are requested one step ahead, right after the previous one has been copied to
+// LDS (one register set of 16).  A wave's loads return in order, so strip p + 1 is requested BEFORE
+// block p + 2.  104 registers less 16 against two full sets: the kernel fits four waves per SIMD,
+// and a launch of about 3300 waves (seq 4096, 16 heads) is resident as a whole.
 // ---------------------------------------------------------------------------
-template <int DEPTH, bool BF>
+template <bool BF>
 __global__ __launch_bounds__(512) void dsd_rows_f16_kernel(
     const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
     const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
@@ -543,93 +547,28 @@ __global__ __launch_bounds__(512) void dsd_rows_f16_kernel(
     const half_t *spb = sp + (sp_shared ? 0 : (size_t)batch * nnz * BS2) + i * BS + 8 * g;
     const half_t *dnb = dn + (size_t)batch * DN * KT + y0;
 
-    struct Frag { uint4 s[2]; uint4 d[4]; };
     DescWindow win;
-    auto load_block = [&](int idx, Frag &f) {
-        const half_t *b = spb + (size_t)idx * BS2;
-        f.s[0] = ldg16_stream(b);
-        f.s[1] = ldg16_stream(b + 16 * BS);
+    uint4 blk[2][2], strip[4];
+    auto issue_block = [&](int p, uint4 (&b)[2]) {             // pair p of a row table names block p
+        const half_t *src = spb + (size_t)p * BS2;
+        b[0] = ldg16_stream(src);
+        b[1] = ldg16_stream(src + 16 * BS);
     };
-    auto load_dense = [&](int p, Frag &f) {
+    auto issue_strip = [&](int p) {
         const half_t *src = dnb + (size_t)(BS * win.get(p).col()) * DN;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int c = l + 64 * q;
-            f.d[q] = ldg16(src + (size_t)(c >> 3) * DN + 8 * (c & 7));
+            strip[q] = ldg16(src + (size_t)(c >> 3) * DN + 8 * (c & 7));
         }
-    };
-    auto load = [&](int p, Frag &f) {
-        load_block(win.get(p).idx, f);
-        load_dense(p, f);
     };
 
     f4v acc[8] = {{0}, {0}, {0}, {0}, {0}, {0}, {0}, {0}};
-    auto compute = [&](const Frag &f) {
-        wave_lds_fence();
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            // rows 8-15 and 24-31 (q odd) are stored with the halves of every piece exchanged
-            const uint4 v = (q & 1) ? make_uint4(f.d[q].z, f.d[q].w, f.d[q].x, f.d[q].y) : f.d[q];
-            *reinterpret_cast<uint4 *>(lds_bytes(tile_d) + put_strip16_addr(l, q)) = v;
-        }
-        wave_lds_fence();
-        h8 dop[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            h4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 0)));
-            h4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 1)));
-            dop[t] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-#pragma unroll
-        for (int xh = 0; xh < 2; ++xh)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) acc[4 * xh + t] = mfma_16x16<BF>(dop[t], as_h8(f.s[xh]), acc[4 * xh + t]);
-    };
-
-    if (e.group >= 0) {
-        Frag fr[DEPTH];
-        for (int seg = e.begin; seg < e.end; seg += WAVE) {
-            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
-            win.fetch(blocks, seg, seg_end);
-            int p = seg;
-            if (seg_end - seg >= 2 * DEPTH) {
-                // steady state without a conditional load; pair p of a row table names block p, so the
-                // first block (from HBM, the longest wait of the wave) does not wait for the descriptors
-                load_block(seg, fr[0]);
-                load_dense(seg, fr[0]);
-#pragma unroll
-                for (int d = 1; d < DEPTH; ++d) load(seg + d, fr[d]);
-                for (; p + 2 * DEPTH <= seg_end; p += DEPTH) {
-#pragma unroll
-                    for (int d = 0; d < DEPTH; ++d) {
-                        compute(fr[d]);
-                        load(p + d + DEPTH, fr[d]);
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int d = 0; d < DEPTH; ++d)
-                    if (seg + d < seg_end) load(seg + d, fr[d]);
-            }
-            for (; p < seg_end; p += DEPTH) {                // the last pairs: loads only while pairs are left
-#pragma unroll
-                for (int d = 0; d < DEPTH; ++d) {
-                    if (p + d < seg_end) {
-                        compute(fr[d]);
-                        if (p + d + DEPTH < seg_end) load(p + d + DEPTH, fr[d]);
-                    }
-                }
-            }
-        }
-    }
-
-    const bool store_it = team_reduce<f4v, 8, 4>(acc, e, w, lds_raw) &&
-                          (e.parts() <= 1 || split_combine<f4v, 8, 4>(acc, e, sched_groups[e.group], ws, batch));
-    if (store_it) {
-        half_t *ob = out + (size_t)batch * XT * DN + y0 + 8 * g;
+    half_t *ob = out + (size_t)batch * XT * DN + y0 + 8 * g;
+    auto store_group = [&](int group) {
 #pragma unroll
         for (int xh = 0; xh < 2; ++xh) {
-            half_t *orow = ob + (size_t)(BS * e.group + 16 * xh + i) * DN;
+            half_t *orow = ob + (size_t)(BS * group + 16 * xh + i) * DN;
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 h8 o;
@@ -641,7 +580,76 @@ __global__ __launch_bounds__(512) void dsd_rows_f16_kernel(
                 stg16(orow + 32 * u, __builtin_bit_cast(uint4, o));
             }
         }
+    };
+
+    auto stage = [&]() {                      // the strip in flight -> LDS
+        wave_lds_fence();
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            // rows 8-15 and 24-31 (q odd) are stored with the halves of every piece exchanged
+            const uint4 v = (q & 1) ? make_uint4(strip[q].z, strip[q].w, strip[q].x, strip[q].y) : strip[q];
+            *reinterpret_cast<uint4 *>(lds_bytes(tile_d) + put_strip16_addr(l, q)) = v;
+        }
+        wave_lds_fence();
+    };
+    auto multiply = [&](const uint4 (&b)[2]) {
+        h8 dop[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            h4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 0)));
+            h4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 1)));
+            dop[t] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int xh = 0; xh < 2; ++xh)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[4 * xh + t] = mfma_16x16<BF>(dop[t], as_h8(b[xh]), acc[4 * xh + t]);
+    };
+
+    if (e.group >= 0) {
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+            issue_block(seg, blk[0]);                 // from HBM, the longest wait: does not wait for the descriptors
+            issue_strip(seg);
+            int p = seg;
+            if (seg + 3 < seg_end) {
+                // steady state, two steps per round.  No load under a condition here nor on the way in: the
+                // compiler's wait counts are only exact when every path into the loop has issued the same loads.
+                issue_block(seg + 1, blk[1]);
+                for (; p + 3 < seg_end; p += 2) {
+                    stage();
+                    issue_strip(p + 1);
+                    multiply(blk[0]);
+                    issue_block(p + 2, blk[0]);
+                    stage();
+                    issue_strip(p + 2);
+                    multiply(blk[1]);
+                    issue_block(p + 3, blk[1]);
+                }
+            } else if (seg + 1 < seg_end) {
+                issue_block(seg + 1, blk[1]);
+            }
+            const int left = seg_end - p;             // 1, 2 or 3 pairs: blocks p and p + 1 and strip p are in flight
+            stage();
+            if (left >= 2) issue_strip(p + 1);
+            multiply(blk[0]);
+            if (left >= 3) issue_block(p + 2, blk[0]);
+            if (left >= 2) {
+                stage();
+                if (left >= 3) issue_strip(p + 2);
+                multiply(blk[1]);
+            }
+            if (left >= 3) {
+                stage();
+                multiply(blk[0]);
+            }
+        }
     }
+
+    const bool store_it = team_reduce<f4v, 8, 4>(acc, e, w, lds_raw) &&
+                          (e.parts() <= 1 || split_combine<f4v, 8, 4>(acc, e, sched_groups[e.group], ws, batch));
+    if (store_it) store_group(e.group);
 }
 
 template <bool S_KC, bool D_KC, bool DSD>
@@ -751,13 +759,6 @@ hipError_t launch_sdd(int dtype, const MatmulArgs &p, hipStream_t st)
     return b_kc ? launch_sdd_f32<false, true>(p, st) : launch_sdd_f32<false, false>(p, st);
 }
 
-// measurement switch while both walks exist: BSA_GW_LEGACY=1 keeps the LDS-staged block
-static bool gw_direct_rows()
-{
-    static const bool on = [] { const char *v = getenv("BSA_GW_LEGACY"); return !(v && v[0] == '1'); }();
-    return on;
-}
-
 template <bool S_KC, bool D_KC, bool DSD>
 static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const MatmulArgs &p,
                               int DN, int KT, int XT, hipStream_t st)
@@ -774,11 +775,11 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
                     sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0, \
                     p.row_table ? 1 : 0
     const bool full = DN % 64 == 0;
-    if (S_KC && !D_KC && DSD && full && p.row_table && dtype != BSA_F32 && gw_direct_rows()) {
+    if (S_KC && !D_KC && DSD && full && p.row_table && dtype != BSA_F32) {
 #define BSA_DR_ARGS (const half_t *)sp, (const half_t *)dn, (half_t *)p.c, (const BlockDesc *)p.blocks, \
                     sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0
-        if (dtype == BSA_F16) dsd_rows_f16_kernel<GW_PREFETCH_DEPTH, false><<<grid, block, lds, st>>>(BSA_DR_ARGS);
-        else dsd_rows_f16_kernel<GW_PREFETCH_DEPTH, true><<<grid, block, lds, st>>>(BSA_DR_ARGS);
+        if (dtype == BSA_F16) dsd_rows_f16_kernel<false><<<grid, block, lds, st>>>(BSA_DR_ARGS);
+        else dsd_rows_f16_kernel<true><<<grid, block, lds, st>>>(BSA_DR_ARGS);
 #undef BSA_DR_ARGS
         return hipGetLastError();
     }

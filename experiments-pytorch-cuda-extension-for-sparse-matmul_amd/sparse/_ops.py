@@ -12,7 +12,7 @@ from . import kernel as _k
 BLOCK = 32
 # tuning of the wavefront schedules: (target pairs per wavefront, wavefronts per workgroup)
 # (cap, waves, split long groups, no row slicing, -, longest chunks first)
-SCHEDULE_GROUP_WALK = (10, 4, True, -1, 2, True)        # groups of at most GROUP_WALK_LONG pairs (rows of attention masks)
+SCHEDULE_GROUP_WALK = (12, 4, True, -1, 2, True)        # groups of at most GROUP_WALK_LONG pairs (rows of attention masks)
 SCHEDULE_GROUP_WALK_LONG = (10, 4, True, -1, 2, True)    # tables with longer groups (columns of causal / strided masks)
 GROUP_WALK_LONG = 24
 SCHEDULE_SDD = (4, 2)
