@@ -255,6 +255,39 @@ int bsa_matmul_noalloc(int mode, int dtype, const void *a, const void *b, void *
 }
 
 
+int bsa_matmul_dsd_block64(int dtype, const void *a, const void *b, void *c,
+                           const int32_t *coarse_row_blocks, const int32_t *coarse_row_offsets,
+                           const int32_t *sched, int sched_wgs, int sched_waves,
+                           int coarse_rows, int coarse_cols, int coarse_nnz, int batches, int sparse_batches,
+                           int N, void *stream)
+{
+    const char *who = "bsa_matmul_dsd_block64";
+    if (dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: fp16 (dtype 1) and bf16 (dtype 2) are built, got %d", who, dtype);
+    if (coarse_rows < 1 || coarse_rows > 16383 || coarse_cols < 1 || coarse_cols > 32767)
+        return fail(BSA_ERR_INVALID, "%s: mask of %d x %d blocks of 64 out of range", who, coarse_rows, coarse_cols);
+    if (coarse_nnz < 0 || (long long)coarse_nnz > (long long)coarse_rows * coarse_cols)
+        return fail(BSA_ERR_INVALID, "%s: %d blocks do not fit a %d x %d mask", who, coarse_nnz, coarse_rows, coarse_cols);
+    if ((long long)coarse_nnz * 4 > 2147483647LL / 2)
+        return fail(BSA_ERR_INVALID, "%s: too many blocks (%d)", who, coarse_nnz);
+    if (batches < 1 || (sparse_batches != batches && sparse_batches != 1))
+        return fail(BSA_ERR_INVALID, "%s: batches %d, sparse_batches %d", who, batches, sparse_batches);
+    if (N < 64 || N % 64)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: the dense width must be a positive multiple of 64, got %d (use bsa_matmul "
+                    "on the expanded tables)", who, N);
+    if (N / 64 > 65535) return fail(BSA_ERR_INVALID, "%s: dense width %d is too large", who, N);
+    if (!c || !b || !coarse_row_offsets || ((!a || !coarse_row_blocks) && coarse_nnz > 0))
+        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    int rc = check_schedule(sched, sched_wgs, sched_waves, batches, who);
+    if (rc) return rc;
+    if (sched_waves > 4)
+        return fail(BSA_ERR_INVALID, "%s: at most 4 waves per workgroup (64 x 64 fp32 tiles meet in LDS), got %d", who,
+                    sched_waves);
+    bsa::Block64Args p{a, b, c, coarse_row_blocks, coarse_row_offsets, sched, coarse_rows, coarse_cols, coarse_nnz,
+                       sched_wgs, sched_waves, batches, N, sparse_batches != batches};
+    return check_launch(bsa::launch_dsd_block64(dtype, p, (hipStream_t)stream), who);
+}
+
 static int check_softmax(const char *who, int dtype, const void *p0, const void *p1, const void *p2,
                          const int32_t *blocks, const int32_t *offsets, const int32_t *sched,
                          int sched_wgs, int sched_waves, int mask_rows, int mask_cols, int nnz, int batches)

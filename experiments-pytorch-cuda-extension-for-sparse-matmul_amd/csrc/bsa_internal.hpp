@@ -43,6 +43,19 @@ hipError_t launch_group_walk(int dtype, bool dsd, const MatmulArgs &p, hipStream
 // the same walk with the split-group workspace in the library's static device buffer (p.workspace is ignored)
 hipError_t launch_group_walk_static_scratch(int dtype, bool dsd, const MatmulArgs &p, hipStream_t stream);
 
+// DSD on a mask of 64 x 64 blocks (coarse tables: one pair per block)
+struct Block64Args {
+    const void *a, *b;
+    void *c;
+    const int32_t *blocks, *offsets;   // row table of the coarse mask
+    const int32_t *sched;              // schedule of that table, built without splitting
+    int coarse_rows, coarse_cols, coarse_nnz;
+    int sched_wgs, sched_waves;
+    int batches, N;
+    bool sparse_shared;
+};
+hipError_t launch_dsd_block64(int dtype, const Block64Args &p, hipStream_t stream);
+
 struct SoftmaxArgs {
     const void *x;    // forward: scores; backward: y
     const void *dy;   // backward only

@@ -9,7 +9,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["api.hip", "layout_build.hip", "matmul.hip", "softmax.hip", "attention.hip", "block_copy.hip"]
-HEADERS = ["bsa_device.hpp", "lds_tiles.hpp", "lds_index_math.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
+HEADERS = ["bench_yardstick.hip", "bsa_device.hpp", "lds_tiles.hpp", "lds_index_math.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
 LIB = os.path.join(HERE, "libbsa_hip.so")
 
 FLAGS = [
@@ -62,7 +62,21 @@ def build(force: bool = False, verbose: bool = False, extra_flags=(), lib: str =
         raise RuntimeError("hipcc failed linking " + os.path.basename(lib))
     if lib == LIB:
         build_index_host(verbose)
+        build_bench_yardstick(verbose)
     return lib
+
+
+def build_bench_yardstick(verbose: bool = False) -> str:
+    """The streaming-copy yardstick bench.py times beside the kernels (its own small library)."""
+    out = os.path.join(HERE, "libbsa_bench.so")
+    cmd = [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")] + FLAGS + [os.path.join(HERE, "bench_yardstick.hip"), "-o", out]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("hipcc failed building libbsa_bench.so")
+    return out
 
 
 def build_index_host(verbose: bool = False) -> str:

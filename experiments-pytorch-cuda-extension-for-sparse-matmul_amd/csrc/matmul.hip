@@ -652,6 +652,152 @@ __global__ __launch_bounds__(512) void dsd_rows_f16_kernel(
     if (store_it) store_group(e.group);
 }
 
+// ---------------------------------------------------------------------------
+// DSD on a mask of 64 x 64 blocks, the block as the unit of work.  The operand is stored as the 2 x 2
+// tiles of 32 x 32 of every block, in the row-major order of the mask with every cell repeated twice
+// along both axes: block j of a coarse row r with n blocks, whose tiles start at base = 4 offsets[r],
+// has its upper tiles at base + 2 j, + 1 and its lower ones 2 n further on.  A wave walks coarse pairs
+// and takes, per 32 columns of the block, the upper and the lower tile (straight into operand registers,
+// as in dsd_rows_f16_kernel) and ONE dense strip, staged once and multiplied into both: 8 KB of strips
+// per 8 KB of block instead of 16 KB when the four tiles are walked as blocks of their own.
+// Accumulators: 64 x 64 fp32 per wave.  Groups are never split across workgroups (the schedule must be
+// built without BSA_SCHED_SPLIT); the waves of a team reduce through LDS.
+// ---------------------------------------------------------------------------
+constexpr int GW64_LDS_PER_WAVE = 16384;    // the strip (4 KB) while walking, the 64 x 64 fp32 partial tile afterwards
+
+template <bool BF>
+__global__ __launch_bounds__(256) void dsd_rows64_f16_kernel(
+    const half_t *__restrict__ sp, const half_t *__restrict__ dn, half_t *__restrict__ out,
+    const BlockDesc *__restrict__ blocks, const int *__restrict__ offsets, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int tiles, int DN, int KT, int XT, int sp_shared)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;   // whole workgroup leaves together
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const int y0 = 64 * (int)blockIdx.y;
+    const int g = l >> 4, i = l & 15;
+
+    half_t *tile_d = reinterpret_cast<half_t *>(lds_raw + (size_t)w * GW64_LDS_PER_WAVE);
+    const half_t *spb = sp + (sp_shared ? 0 : (size_t)batch * tiles * BS2) + i * BS + 8 * g;
+    const half_t *dnb = dn + (size_t)batch * DN * KT + y0;
+
+    f4v acc[16];                       // acc[8 r + 4 xh + t]: tile row r (upper, lower), 16 block rows xh, columns col16(t, .)
+#pragma unroll
+    for (int t = 0; t < 16; ++t) acc[t] = f4v{0};
+
+    if (e.group >= 0 && e.begin < e.end) {
+        const int first = offsets[e.group], n = offsets[e.group + 1] - first;
+        const size_t upper = (size_t)4 * first, lower = upper + (size_t)2 * n;      // tile index of column step 0
+        DescWindow win;
+        uint4 blk[2][4], strip[4];
+        // column step s = 2 (pair - first) + half: the 32 columns `half` of the pair's block
+        auto issue_block = [&](int s, uint4 (&b)[4]) {
+            const half_t *up = spb + (upper + s) * BS2, *lo = spb + (lower + s) * BS2;
+            b[0] = ldg16_stream(up);
+            b[1] = ldg16_stream(up + 16 * BS);
+            b[2] = ldg16_stream(lo);
+            b[3] = ldg16_stream(lo + 16 * BS);
+        };
+        auto issue_strip = [&](int s) {
+            const int col32 = 2 * win.get(first + (s >> 1)).col() + (s & 1);
+            const half_t *src = dnb + (size_t)(BS * col32) * DN;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int c = l + 64 * q;
+                strip[q] = ldg16(src + (size_t)(c >> 3) * DN + 8 * (c & 7));
+            }
+        };
+        auto stage = [&]() {
+            wave_lds_fence();
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint4 v = (q & 1) ? make_uint4(strip[q].z, strip[q].w, strip[q].x, strip[q].y) : strip[q];
+                *reinterpret_cast<uint4 *>(lds_bytes(tile_d) + put_strip16_addr(l, q)) = v;
+            }
+            wave_lds_fence();
+        };
+        auto multiply = [&](const uint4 (&b)[4]) {
+            h8 dop[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                h4 lo = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 0)));
+                h4 hi = lds_read_tr16(reinterpret_cast<const half_t *>(lds_bytes(tile_d) + get_strip16_addr(l, t, 1)));
+                dop[t] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int xh = 0; xh < 2; ++xh)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        acc[8 * r + 4 * xh + t] = mfma_16x16<BF>(dop[t], as_h8(b[2 * r + xh]), acc[8 * r + 4 * xh + t]);
+        };
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+            int s = 2 * (seg - first);
+            const int s_end = 2 * (seg_end - first), last = s_end - 1;     // an even number of column steps
+            issue_block(s, blk[0]);
+            issue_strip(s);
+            issue_block(s + 1, blk[1]);
+            // Two steps per round and no load under a condition: behind the last step the requests repeat it
+            // (served by the caches, never used), which keeps ONE copy of the loop body and exact wait counts.
+            for (; s < s_end; s += 2) {
+                stage();
+                issue_strip(s + 1);
+                multiply(blk[0]);
+                issue_block(s + 2 < last ? s + 2 : last, blk[0]);
+                stage();
+                issue_strip(s + 2 < last ? s + 2 : last);
+                multiply(blk[1]);
+                issue_block(s + 3 < last ? s + 3 : last, blk[1]);
+            }
+        }
+    }
+
+    // team reduction through LDS: every wave of the workgroup arrives here once
+    const int slot0 = e.first_wave(), nw = e.team_waves();
+    const bool active = e.group >= 0;
+    const bool leader = active && w == slot0;
+    float *mine = reinterpret_cast<float *>(lds_raw + (size_t)w * GW64_LDS_PER_WAVE);
+    if (active && !leader) {
+        wave_lds_fence();
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) mine[(t * 4 + v) * WAVE + l] = acc[t][v];
+    }
+    __syncthreads();
+    if (!leader) return;
+    for (int o = 1; o < nw; ++o) {
+        const float *other = reinterpret_cast<const float *>(lds_raw + (size_t)(w + o) * GW64_LDS_PER_WAVE);
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[t][v] += other[(t * 4 + v) * WAVE + l];
+    }
+    half_t *ob = out + (size_t)batch * XT * DN + y0 + 8 * g;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int xh = 0; xh < 2; ++xh) {
+            half_t *orow = ob + (size_t)(64 * e.group + 32 * r + 16 * xh + i) * DN;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                h8 o;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    o[v] = narrow_16<BF>(acc[8 * r + 4 * xh + 2 * u][v]);
+                    o[4 + v] = narrow_16<BF>(acc[8 * r + 4 * xh + 2 * u + 1][v]);
+                }
+                stg16(orow + 32 * u, __builtin_bit_cast(uint4, o));
+            }
+        }
+}
+
 template <bool S_KC, bool D_KC, bool DSD>
 __global__ __launch_bounds__(512) void gw_f32_kernel(
     const float *__restrict__ sp, const float *__restrict__ dn, float *__restrict__ out,
@@ -794,6 +940,30 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
         gw_f32_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(
             (const float *)sp, (const float *)dn, (float *)p.c, (const BlockDesc *)p.blocks,
             sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
+    return hipGetLastError();
+}
+
+hipError_t launch_dsd_block64(int dtype, const Block64Args &p, hipStream_t st)
+{
+    dim3 grid(grid_x(p.sched_wgs, p.batches), (unsigned)(p.N / 64)), block(64 * p.sched_waves);
+    const size_t lds = (size_t)p.sched_waves * GW64_LDS_PER_WAVE;
+    const SchedEntry *slots = (const SchedEntry *)p.sched + p.coarse_rows;
+    hipError_t err = hipSuccess;
+    if (dtype == BSA_F16) {
+        if (lds > 65536) err = hipFuncSetAttribute(reinterpret_cast<const void *>(dsd_rows64_f16_kernel<false>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+        dsd_rows64_f16_kernel<false><<<grid, block, lds, st>>>(
+            (const half_t *)p.a, (const half_t *)p.b, (half_t *)p.c, (const BlockDesc *)p.blocks, p.offsets, slots,
+            p.sched_wgs, p.batches, 4 * p.coarse_nnz, p.N, 64 * p.coarse_cols, 64 * p.coarse_rows, p.sparse_shared ? 1 : 0);
+    } else {
+        if (lds > 65536) err = hipFuncSetAttribute(reinterpret_cast<const void *>(dsd_rows64_f16_kernel<true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+        dsd_rows64_f16_kernel<true><<<grid, block, lds, st>>>(
+            (const half_t *)p.a, (const half_t *)p.b, (half_t *)p.c, (const BlockDesc *)p.blocks, p.offsets, slots,
+            p.sched_wgs, p.batches, 4 * p.coarse_nnz, p.N, 64 * p.coarse_cols, 64 * p.coarse_rows, p.sparse_shared ? 1 : 0);
+    }
     return hipGetLastError();
 }
 

@@ -20,6 +20,12 @@ SCHEDULE_SDD_F32 = (1, 4)              # fp32 SDD reloads both operands per bloc
 SCHEDULE_SOFTMAX = (4, 4)
 SOFTMAX_LONGEST_FIRST = True     # long rows are dispatched first: they would otherwise finish on a draining machine
 SOFTMAX_WAVES_LONG_ROWS = 8
+SCHEDULE_BLOCK64 = (4, 2, False)        # coarse pairs (64x64 blocks = four tiles) per wavefront; never split
+# DSD on a block=64 layout: True takes the kernel whose wavefronts own whole 64x64 blocks, False walks the layout's
+# 32x32 tiles.  Measured at 4096 tokens, 16 heads, 399 blocks of 64 (bench.py, rows block64_mask_*): 18.8 us against
+# 17.1 us; a wavefront that holds a 64 x 64 fp32 tile needs 227 registers (two waves per SIMD), so the tile walk stays
+# the default.
+USE_BLOCK64_KERNEL = False
 ATTENTION_WAVES_LONG_GROUPS = 8
 ATTENTION_SPLIT_ROWS = True       # groups longer than cap * waves are cut into parts across workgroups
 SCHEDULE_ATTENTION = (12, 4)           # forward: rows of more than 48 blocks are split across workgroups
@@ -219,6 +225,18 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
     else:
         shape = batch_a + (num_blocks, BLOCK, BLOCK)
     c = torch.empty(shape, dtype=a.dtype, device=a.device)
+
+    coarse = getattr(row_layout[1], "_bsa_coarse", None)
+    if (USE_BLOCK64_KERNEL and coarse is not None and mode == "dsd" and not trans_a and not trans_b
+            and a.dtype != torch.float32 and size_n % 64 == 0 and num_blocks > 0):
+        (cblocks, coffsets), crows, ccols = coarse
+        sched = schedule_for((cblocks, coffsets), SCHEDULE_BLOCK64)
+        with torch.cuda.device(a.device):
+            _k.check(_k.lib.bsa_matmul_dsd_block64(
+                _DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), c.data_ptr(), cblocks.data_ptr(), coffsets.data_ptr(),
+                sched.table.data_ptr(), sched.workgroups, sched.waves, crows, ccols, cblocks.numel() // 2, batches,
+                1 if shared else batches, size_n, _k.current_stream()))
+        return c
 
     if mode == "sdd":
         sched = schedule_for(layout, SCHEDULE_SDD_F32 if a.dtype == torch.float32 else SCHEDULE_SDD)

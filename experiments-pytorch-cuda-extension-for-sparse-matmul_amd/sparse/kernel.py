@@ -34,6 +34,7 @@ SIGNATURES = {
                         _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "bsa_matmul_noalloc": (_i, [_i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i,
                                 _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "bsa_matmul_dsd_block64": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "bsa_softmax_forward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "bsa_softmax_backward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
     "bsa_to_sparse": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),

@@ -11,9 +11,12 @@ memory, other dtypes) take a torch gather; a bool mask means the same as the 0/1
 integer mask.
 
 ``block=64`` (not in the reference, whose kernels are 32x32x32 only) accepts a mask of
-64x64 blocks: every kept block is run as its 2x2 tiles of 32x32, i.e. the tables, the
-block stack ``[..., 4 * kept, 32, 32]`` and every kernel are those of the mask with each
-cell repeated twice along both axes.  No kernel treats a 64x64 block as a unit.
+64x64 blocks: the tables and the block stack ``[..., 4 * kept, 32, 32]`` are those of the
+mask with each cell repeated twice along both axes, and every operator can run on them as
+on any 32x32 layout.  The layout also keeps the row table of the coarse mask
+(``coarse_row_layout``, attached to the row offsets so that it travels with the tables
+through ``sparse_ops.sparse_matmul``): the untransposed fp16 / bf16 DSD product takes it to
+``bsa_matmul_dsd_block64``, whose wavefronts own whole 64x64 blocks.
 """
 from typing import Tuple
 
@@ -80,6 +83,23 @@ class SparseLayout:
         # exact-size tensors: the boundary derives nnz from blocks.size(0) / 2 (sparse_kernels.cc:13)
         self.row_layout: Tuple[torch.Tensor, torch.Tensor] = (row_blocks[:2 * nnz].clone(), row_offsets)
         self.col_layout: Tuple[torch.Tensor, torch.Tensor] = (col_blocks[:2 * nnz].clone(), col_offsets)
+
+        self.coarse_row_layout = None
+        if per_side > 1:
+            # row table of the mask in 64x64 blocks, for the kernel that owns whole blocks
+            cmask = (pattern != 0).to(device=self.device, dtype=torch.uint8).contiguous()
+            crows, ccols = cmask.shape
+            cb = torch.empty(2 * crows * ccols, dtype=torch.int32, device=self.device)
+            cb2 = torch.empty_like(cb)
+            co = torch.empty(crows + 1, dtype=torch.int32, device=self.device)
+            co2 = torch.empty(ccols + 1, dtype=torch.int32, device=self.device)
+            cws = torch.empty(_k.lib.bsa_layout_workspace_bytes(crows, ccols), dtype=torch.uint8, device=self.device)
+            with torch.cuda.device(self.device):
+                _k.check(_k.lib.bsa_layout_build(cmask.data_ptr(), crows, ccols, cb.data_ptr(), co.data_ptr(),
+                                                 cb2.data_ptr(), co2.data_ptr(), nnz_dev.data_ptr(), cws.data_ptr(),
+                                                 _k.current_stream()))
+            self.coarse_row_layout = (cb[:nnz // 2].clone(), co)
+            self.row_layout[1]._bsa_coarse = (self.coarse_row_layout, crows, ccols)
 
         packed = self.row_layout[0].view(-1, 2)[:, 1].long()
         # [nnz, 2] (row, col) in row-major order == torch.nonzero(pattern) (layout.py:8)

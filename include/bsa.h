@@ -196,6 +196,27 @@ int bsa_matmul_noalloc(int mode, int dtype, const void *a, const void *b, void *
                        int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
                        int M, int N, int K, int tr_a, int tr_b, void *stream);
 
+/* ---- DSD on a mask of 64x64 blocks, the block as the unit of work -------------
+ * No counterpart in the reference, whose kernels are 32x32x32 only (sparse/native/sparse_smm_gpu.cu:22,
+ * :106, :192, and the hard-coded 32 of sparse/layout.py:42-45).  c[b] = S(a)[b] * b[b] for a sparse
+ * operand whose mask is given in blocks of 64: a wavefront owns whole 64 x 64 blocks, so a dense strip
+ * of 32 x 64 is fetched and staged once for the upper and the lower half of a block (half the strip
+ * traffic of bsa_matmul on the same mask expanded to 32 x 32 tiles, same results).
+ *   a        [sparse_batches, 4 * coarse_nnz, 32, 32]: the 2 x 2 tiles of every block, in the row-major
+ *            order of the mask with every cell repeated twice along both axes (what bsa_layout_build /
+ *            bsa_to_sparse give for that expanded mask); sparse_batches = batches, or 1 (shared)
+ *   b        [batches, 64 * coarse_cols, N], c [batches, 64 * coarse_rows, N], N a multiple of 64
+ *   coarse_row_blocks / coarse_row_offsets: the ROW table of the coarse mask (one pair per block)
+ *   sched    schedule of that table from bsa_schedule_build WITHOUT BSA_SCHED_SPLIT and with at most
+ *            4 waves per workgroup (a group never leaves its workgroup; no workspace is needed)
+ * fp16 / bf16, no transposes; everything else goes through bsa_matmul on the expanded tables.
+ */
+int bsa_matmul_dsd_block64(int dtype, const void *a, const void *b, void *c,
+                           const int32_t *coarse_row_blocks, const int32_t *coarse_row_offsets,
+                           const int32_t *sched, int sched_wgs, int sched_waves,
+                           int coarse_rows, int coarse_cols, int coarse_nnz, int batches, int sparse_batches,
+                           int N, void *stream);
+
 /* ---- block-sparse softmax ----------------------------------------------
  * Replaces sparse_softmax_forward / sparse_softmax_backward
  * (sparse_softmax.cu:208-258) and their kernels (:113-205), with two additions:

@@ -71,3 +71,55 @@ def test_operators_on_64_blocks(name, mask):
                       mo.matmul(v.numpy(), p.float().cpu().numpy(), "dds", tiles, True, False)) <= FP16_TOL
     fused = sparse.attention(q.cuda(), k.cuda(), v.cuda(), L, 0.125, True)
     assert mo.rel_err(fused.float().cpu().numpy(), ao.forward(q.numpy(), k.numpy(), v.numpy(), tiles, 0.125, True)) <= FP16_TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name,mask", _masks() + [("long_rows_3x40", np.ones((3, 40), dtype=np.int64))])
+def test_dsd_kernel_that_owns_whole_blocks(name, mask, dtype):
+    """The untransposed DSD product on a block=64 layout goes to bsa_matmul_dsd_block64 (a wavefront owns
+    64 x 64 blocks, one dense strip serves the upper and the lower tiles): against the oracle on the
+    expanded mask, against the walk over 32 x 32 tiles of the same layout, with one sparse operand shared
+    by the batch, and with a dense width of 128."""
+    import sparse
+    from sparse import _ops
+    L = sparse.SparseLayout(torch.as_tensor(mask), block=64)
+    assert L.coarse_row_layout is not None and L.coarse_row_layout[0].numel() == 2 * int(mask.sum())
+    tiles = _expand(mask)
+    g = torch.Generator().manual_seed(64 + mask.shape[1])
+    tol = FP16_TOL if dtype == torch.float16 else 1e-2
+    for width, batch in ((64, 3), (128, 2)):
+        s = torch.rand(batch, L.num_blocks, 32, 32, generator=g).to(dtype)
+        v = torch.randn(batch, 64 * mask.shape[1], width, generator=g).to(dtype)
+        ref = mo.matmul(s.float().numpy().astype(np.float64), v.float().numpy().astype(np.float64), "dsd", tiles)
+        calls = []
+        real = sparse.kernel.lib.bsa_matmul_dsd_block64
+        _ops.USE_BLOCK64_KERNEL = True
+        try:
+            sparse.kernel.lib.bsa_matmul_dsd_block64 = lambda *a: (calls.append(1), real(*a))[1]
+            out = sparse.matmul(s.cuda(), v.cuda(), "dsd", L)
+        finally:
+            sparse.kernel.lib.bsa_matmul_dsd_block64 = real
+            _ops.USE_BLOCK64_KERNEL = False
+        assert calls, "the 64 x 64 kernel was not taken"
+        assert mo.rel_err(out.float().cpu().numpy(), ref) <= tol
+        by_tiles = sparse.matmul(s.cuda(), v.cuda(), "dsd", L)
+        assert mo.rel_err(out.float().cpu().numpy(), by_tiles.float().cpu().numpy().astype(np.float64)) <= tol
+    # one sparse operand for the whole batch
+    s1 = torch.rand(L.num_blocks, 32, 32, generator=g).to(dtype)
+    v = torch.randn(2, 64 * mask.shape[1], 64, generator=g).to(dtype)
+    _ops.USE_BLOCK64_KERNEL = True
+    try:
+        out = sparse.matmul(s1.cuda(), v.cuda(), "dsd", L)
+    finally:
+        _ops.USE_BLOCK64_KERNEL = False
+    ref = mo.matmul(s1.expand(2, -1, -1, -1).float().numpy().astype(np.float64), v.float().numpy().astype(np.float64), "dsd", tiles)
+    assert mo.rel_err(out.float().cpu().numpy(), ref) <= tol
+    # gradients still flow (the backward products take the tile walks)
+    sd = torch.rand(1, L.num_blocks, 32, 32, generator=g).to(dtype).cuda().requires_grad_(True)
+    vd = torch.randn(1, 64 * mask.shape[1], 64, generator=g).to(dtype).cuda().requires_grad_(True)
+    _ops.USE_BLOCK64_KERNEL = True
+    try:
+        sparse.matmul(sd, vd, "dsd", L).float().sum().backward()
+    finally:
+        _ops.USE_BLOCK64_KERNEL = False
+    assert sd.grad is not None and vd.grad is not None and torch.isfinite(sd.grad).all() and torch.isfinite(vd.grad).all()
