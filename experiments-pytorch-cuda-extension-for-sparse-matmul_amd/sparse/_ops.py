@@ -62,45 +62,67 @@ class Schedule:
         self.cap = cap
         self._workspaces = {}
         self._spares = {}
+        self.last_key = None
 
     def workspace(self, mode: int, batches: int, size_m: int, size_n: int, stream: int):
         """Zeroed scratch for split groups, one per (shape, stream): launches on one stream run in
         order and each leaves the buffer zero again; launches on different streams may overlap."""
         need = _k.lib.bsa_matmul_workspace_bytes(mode, self.tile_slots, self.split_groups, batches, size_m, size_n)
-        return self._zeroed((mode, batches, size_m, size_n, stream), need)
+        self.last_key = (mode, batches, size_m, size_n, stream)
+        return self._zeroed(self.last_key, need)
 
     def attention_workspace(self, batches: int, head_dim: int, stream: int):
         """The same for the split rows of the fused attention forward."""
         need = _k.lib.bsa_attention_workspace_bytes(self.tile_slots, self.split_groups, batches, head_dim)
-        return self._zeroed(("attention", batches, head_dim, stream), need)
+        self.last_key = ("attention", batches, head_dim, stream)
+        return self._zeroed(self.last_key, need)
 
     def attention_backward_workspace(self, columns, batches: int, head_dim: int, stream: int):
         """The same for the backward walks: this schedule walks the rows, ``columns`` (or None) the columns."""
         ct, cg = (columns.tile_slots, columns.split_groups) if columns is not None else (0, 0)
         need = _k.lib.bsa_attention_backward_workspace_bytes(self.tile_slots, self.split_groups, ct, cg, batches,
                                                              head_dim)
-        return self._zeroed(("attention_backward", id(columns), batches, head_dim, stream), need)
+        self.last_key = ("attention_backward", id(columns), batches, head_dim, stream)
+        return self._zeroed(self.last_key, need)
+
+    MAX_WORKSPACES = 16      # per schedule; the least recently used one goes first
 
     def _zeroed(self, key, need):
         """Workspace of ``need`` zero bytes for ``key`` (its last item is the stream).  A buffer must be
         zero before its first launch, and under graph capture nothing can be zeroed (a fill recorded
-        there only runs at replay, possibly after another graph has used the buffer): the first eager
-        call for a shape therefore prepares a second buffer, which a capture on another stream takes."""
+        there only runs at replay, possibly after another graph has used the buffer): every eager call
+        keeps one zeroed spare per shape ready, which a first use under capture takes."""
         if need == 0:
             return None, 0
-        ws = self._workspaces.get(key)
+        ws = self._workspaces.pop(key, None)
+        capturing = torch.cuda.is_current_stream_capturing()
+        spares = self._spares.setdefault(key[:-1], [])
         if ws is None:
-            spares = self._spares.setdefault(key[:-1], [])
-            if torch.cuda.is_current_stream_capturing():
+            if capturing:
                 if not spares:
-                    raise RuntimeError("first use of this operator and shape under graph capture: call it once "
+                    raise RuntimeError("this operator and shape has never run outside graph capture: call it once "
                                        "eagerly before capturing (its workspace must be zeroed first)")
                 ws = spares.pop()
             else:
                 ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
-                spares.append(torch.zeros(need, dtype=torch.uint8, device=self.table.device))
-            self._workspaces[key] = ws
+        if not capturing and not spares:
+            spares.append(torch.zeros(need, dtype=torch.uint8, device=self.table.device))
+        self._workspaces[key] = ws                      # most recently used last
+        while len(self._workspaces) > self.MAX_WORKSPACES:
+            self._workspaces.pop(next(iter(self._workspaces)))
         return ws, need
+
+    def discard(self, key):
+        """Forget the workspace of ``key``: a launch that failed may have left its counters non-zero."""
+        self._workspaces.pop(key, None)
+
+
+def _launch(sched, status):
+    """Raise on a failed C-ABI call; the workspace the call was given is dropped first, because a launch
+    that failed midway may have left its counters non-zero and every later call would sum stale parts."""
+    if status != 0 and sched is not None and sched.last_key is not None:
+        sched.discard(sched.last_key)
+    _k.check(status)
 
 
 def schedule_for(layout, kind):
@@ -131,9 +153,9 @@ def _group_walk_schedule(layout):
 
 
 def _attention_schedule(layout, kind, split=False):
-    """Schedule of a fused attention walk.  The backward walks never split a group across workgroups,
-    so a table with a group longer than the workgroup's share gets the most waves a workgroup holds;
-    the forward walk (``split``) cuts such a row into parts that meet in a workspace."""
+    """Schedule of a fused attention walk.  With ``split`` (what every caller passes while
+    ``ATTENTION_SPLIT_ROWS`` is set) a group longer than the workgroup's share is cut into parts that
+    meet in a workspace; without it such a table gets the most waves a workgroup holds instead."""
     cap, waves = kind
     if split:
         return schedule_for(layout, (cap, waves, True))
@@ -245,7 +267,7 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
     with torch.cuda.device(a.device):
         stream = _k.current_stream()
         ws, ws_bytes = sched.workspace(_k.MODES[mode], batches, size_m, size_n, stream)
-        _k.check(_k.lib.bsa_matmul(
+        _launch(sched, _k.lib.bsa_matmul(
             _k.MODES[mode], _DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), c.data_ptr(),
             layout[0].data_ptr(), layout[1].data_ptr(), layout[1].numel() - 1,
             sched.table.data_ptr(), sched.workgroups, sched.waves, sched.tile_slots, sched.split_groups,
@@ -348,7 +370,7 @@ def sparse_attention_forward(q, k, v, row_blocks, row_table, scale=1.0, causal=F
         with torch.cuda.device(q.device):
             stream = _k.current_stream()
             ws, ws_bytes = sched.attention_workspace(batches, head, stream)
-            _k.check(_k.lib.bsa_attention_forward(
+            _launch(sched, _k.lib.bsa_attention_forward(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                 lse.data_ptr() if lse is not None else None,
                 row_blocks.data_ptr(), row_table.data_ptr(), sched.table.data_ptr(), sched.workgroups, sched.waves,
@@ -379,7 +401,7 @@ def sparse_attention_backward_scores(q, k, v, dout, out, lse, row_blocks, row_ta
         with torch.cuda.device(q.device):
             stream = _k.current_stream()
             ws, ws_bytes = sched.attention_backward_workspace(None, batches, head, stream) if with_dq else (None, 0)
-            _k.check(_k.lib.bsa_attention_backward_scores(
+            _launch(sched, _k.lib.bsa_attention_backward_scores(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
                 lse.data_ptr(), p.data_ptr(), ds.data_ptr(), dq.data_ptr() if with_dq else None,
                 row_blocks.data_ptr(), row_table.data_ptr(),
@@ -414,7 +436,7 @@ def sparse_attention_backward(q, k, v, dout, out, lse, row_blocks, row_table, co
         with torch.cuda.device(q.device):
             stream = _k.current_stream()
             ws, ws_bytes = rs.attention_backward_workspace(cs, batches, head, stream)
-            _k.check(_k.lib.bsa_attention_backward(
+            _launch(rs, _k.lib.bsa_attention_backward(
                 _DTYPES[q.dtype], q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), out.data_ptr(),
                 lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(),
                 row_blocks.data_ptr(), row_table.data_ptr(), rs.table.data_ptr(), rs.workgroups, rs.waves,
