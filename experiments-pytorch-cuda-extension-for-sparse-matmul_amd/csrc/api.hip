@@ -288,6 +288,67 @@ int bsa_matmul_dsd_block64(int dtype, const void *a, const void *b, void *c,
     return check_launch(bsa::launch_dsd_block64(dtype, p, (hipStream_t)stream), who);
 }
 
+int64_t bsa_run_schedule_bytes(int mask_rows, int nnz)
+{
+    if (mask_rows < 1 || nnz < 0) return 0;
+    return (int64_t)mask_rows * bsa::RUN_RECORD_BYTES + (((int64_t)nnz + 3) & ~(int64_t)3);
+}
+
+int bsa_run_schedule_build(const int32_t *row_blocks, const int32_t *row_offsets, int mask_rows, int nnz,
+                           int target_pairs, int max_strips, void *sched, int64_t sched_bytes,
+                           int32_t *counts_out, void *stream)
+{
+    const char *who = "bsa_run_schedule_build";
+    if (mask_rows < 1 || mask_rows > 32767) return fail(BSA_ERR_INVALID, "%s: %d block rows outside [1, 32767]", who, mask_rows);
+    if (nnz < 0) return fail(BSA_ERR_INVALID, "%s: nnz %d < 0", who, nnz);
+    if (target_pairs < 1) return fail(BSA_ERR_INVALID, "%s: target_pairs %d < 1", who, target_pairs);
+    if (max_strips < 1 || max_strips > bsa::RUN_MAX_STRIPS)
+        return fail(BSA_ERR_INVALID, "%s: max_strips %d outside [1, %d]", who, max_strips, bsa::RUN_MAX_STRIPS);
+    if (!row_offsets || !sched || !counts_out || (!row_blocks && nnz > 0))
+        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if (sched_bytes < bsa_run_schedule_bytes(mask_rows, nnz))
+        return fail(BSA_ERR_INVALID, "%s: the schedule needs %lld bytes, got %lld", who,
+                    (long long)bsa_run_schedule_bytes(mask_rows, nnz), (long long)sched_bytes);
+    return check_launch(bsa::launch_run_schedule_build(row_blocks, row_offsets, mask_rows, nnz, target_pairs, max_strips,
+                                                       sched, counts_out, (hipStream_t)stream), who);
+}
+
+int bsa_matmul_dsd_runs(int dtype, const void *a, const void *b, void *c,
+                        const int32_t *row_blocks, const int32_t *row_offsets,
+                        const void *run_sched, int n_runs, int run_strips, int run_pairs, int waves,
+                        int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
+                        int N, void *stream)
+{
+    const char *who = "bsa_matmul_dsd_runs";
+    if (dtype != BSA_F16 && dtype != BSA_BF16)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: fp16 (dtype 1) and bf16 (dtype 2) are built, got %d", who, dtype);
+    if (mask_rows < 1 || mask_rows > 32767 || mask_cols < 1 || mask_cols > 65535)
+        return fail(BSA_ERR_INVALID, "%s: mask shape %d x %d out of range", who, mask_rows, mask_cols);
+    if (nnz < 0 || (long long)nnz > (long long)mask_rows * mask_cols)
+        return fail(BSA_ERR_INVALID, "%s: nnz %d does not fit a %d x %d mask", who, nnz, mask_rows, mask_cols);
+    if (batches < 1 || (sparse_batches != batches && sparse_batches != 1))
+        return fail(BSA_ERR_INVALID, "%s: batches %d, sparse_batches %d", who, batches, sparse_batches);
+    if (N < 64 || N % 64)
+        return fail(BSA_ERR_UNSUPPORTED, "%s: the dense width must be a positive multiple of 64, got %d (use bsa_matmul)", who, N);
+    if (N / 64 > 65535) return fail(BSA_ERR_INVALID, "%s: dense width %d is too large", who, N);
+    if (!c || !b || !row_offsets || !run_sched || ((!a || !row_blocks) && nnz > 0))
+        return fail(BSA_ERR_INVALID, "%s: null pointer argument", who);
+    if (n_runs < 1 || n_runs > mask_rows)
+        return fail(BSA_ERR_INVALID, "%s: %d runs for %d block rows (a table that bsa_run_schedule_build reports as not "
+                    "eligible has none: use bsa_matmul)", who, n_runs, mask_rows);
+    if (waves < 1 || waves > bsa::RUN_MAX_WAVES)
+        return fail(BSA_ERR_INVALID, "%s: %d waves per workgroup outside [1, %d]", who, waves, bsa::RUN_MAX_WAVES);
+    if (run_strips < 0 || run_strips > bsa::RUN_MAX_STRIPS || run_strips > 4 * waves)
+        return fail(BSA_ERR_INVALID, "%s: %d strips per run: at most %d, and 4 per wave", who, run_strips, bsa::RUN_MAX_STRIPS);
+    if (run_pairs < 0 || run_pairs > 64 * waves)
+        return fail(BSA_ERR_INVALID, "%s: a run of %d pairs needs more than %d waves (64 pairs each)", who, run_pairs, waves);
+    if ((long long)n_runs * ((batches + 7) / 8) > (1LL << 27))
+        return fail(BSA_ERR_INVALID, "%s: %d runs x %d batch entries do not fit one launch", who, n_runs, batches);
+    bsa::RunsArgs p{a, b, c, row_blocks, row_offsets, run_sched, n_runs, waves, run_strips < 1 ? 1 : run_strips,
+                    mask_rows, mask_cols, nnz, batches, N, sparse_batches != batches};
+    return check_launch(bsa::launch_dsd_runs(dtype, p, (hipStream_t)stream), who);
+}
+
 static int check_softmax(const char *who, int dtype, const void *p0, const void *p1, const void *p2,
                          const int32_t *blocks, const int32_t *offsets, const int32_t *sched,
                          int sched_wgs, int sched_waves, int mask_rows, int mask_cols, int nnz, int batches)

@@ -56,6 +56,25 @@ struct Block64Args {
 };
 hipError_t launch_dsd_block64(int dtype, const Block64Args &p, hipStream_t stream);
 
+// DSD over runs of block rows with the dense strips of a run resident in LDS (dsd_runs.hip)
+constexpr int RUN_RECORD_BYTES = 160;      // one record per run; the schedule is [records x mask rows][one byte per pair]
+constexpr int RUN_MAX_STRIPS = 39;         // 4 KB each, next to the per-wave flags, in the 160 KB of a compute unit
+constexpr int RUN_MAX_WAVES = 12;
+hipError_t launch_run_schedule_build(const int32_t *row_blocks, const int32_t *row_offsets, int rows, int nnz,
+                                     int target_pairs, int max_strips, void *sched, int32_t *counts_out,
+                                     hipStream_t stream);
+struct RunsArgs {
+    const void *a, *b;
+    void *c;
+    const int32_t *blocks, *offsets;   // row table
+    const void *sched;                 // run schedule of that table
+    int n_runs, waves, strips;         // strips: the widest run's (counts_out[1] of the build)
+    int mask_rows, mask_cols, nnz;
+    int batches, N;
+    bool sparse_shared;
+};
+hipError_t launch_dsd_runs(int dtype, const RunsArgs &p, hipStream_t stream);
+
 struct SoftmaxArgs {
     const void *x;    // forward: scores; backward: y
     const void *dy;   // backward only

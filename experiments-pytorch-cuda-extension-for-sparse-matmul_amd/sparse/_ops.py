@@ -26,6 +26,20 @@ SCHEDULE_BLOCK64 = (4, 2, False)        # coarse pairs (64x64 blocks = four tile
 # 17.1 us; a wavefront that holds a 64 x 64 fp32 tile needs 227 registers (two waves per SIMD), so the tile walk stays
 # the default.
 USE_BLOCK64_KERNEL = False
+# DSD over a row table with the dense operand stored [K][N]: runs of consecutive block rows whose dense strips stay
+# in LDS (bsa_matmul_dsd_runs), when the table is eligible, a fetched strip serves at least RUN_WALK_MIN_REUSE pairs
+# and the launch is large enough to give every compute unit a run of RUN_WALK_PAIRS_MIN pairs.  A run is one
+# workgroup with a compute unit to itself; the launch is cut into a whole number of generations of about
+# RUN_WALK_PAIRS pairs per run (workgroups a few above a multiple of the compute units would cost a generation of
+# their own).  Measured at 4096 tokens (1530 blocks per head), DSD fp16, against the walk of bsa_matmul:
+# 10.2 / 10.8 / 16.1 / 24.3 / 29.4 / 42.0 us against 12.3 / 12.9 / 16.9 / 26.1 / 33.5 / 44.8 us at
+# 4 / 8 / 16 / 24 / 32 / 48 heads.
+RUN_WALK = True
+RUN_WALK_WAVES = 8               # more (4 strips per wave) only for runs of more than 32 strips
+RUN_WALK_PAIRS = 96
+RUN_WALK_PAIRS_MIN = 48
+RUN_WALK_STRIPS = 39
+RUN_WALK_MIN_REUSE = 2.0
 ATTENTION_WAVES_LONG_GROUPS = 8
 ATTENTION_SPLIT_ROWS = True       # groups longer than cap * waves are cut into parts across workgroups
 SCHEDULE_ATTENTION = (12, 4)           # forward: rows of more than 48 blocks are split across workgroups
@@ -115,6 +129,55 @@ class Schedule:
     def discard(self, key):
         """Forget the workspace of ``key``: a launch that failed may have left its counters non-zero."""
         self._workspaces.pop(key, None)
+
+
+class RunSchedule:
+    """Runs of consecutive block rows of a row table (bsa_run_schedule_build)."""
+
+    def __init__(self, blocks: torch.Tensor, offsets: torch.Tensor, target_pairs: int, max_strips: int):
+        rows, nnz = offsets.numel() - 1, blocks.numel() // 2
+        need = _k.lib.bsa_run_schedule_bytes(rows, nnz)
+        self.table = torch.empty(need, dtype=torch.uint8, device=offsets.device)
+        counts = torch.empty(4, dtype=torch.int32, device=offsets.device)
+        with torch.cuda.device(offsets.device):
+            _k.check(_k.lib.bsa_run_schedule_build(blocks.data_ptr(), offsets.data_ptr(), rows, nnz, target_pairs,
+                                                   max_strips, self.table.data_ptr(), need, counts.data_ptr(),
+                                                   _k.current_stream()))
+        self.runs, self.strips, self.strips_total, self.pairs = (int(v) for v in counts.tolist())
+        self.reuse = nnz / self.strips_total if self.strips_total else 0.0
+
+
+def _run_schedule(layout, batches, strips_n):
+    """Run schedule of a row table for a launch of ``batches`` x ``strips_n`` (64-column strips of the result)
+    entries, or None when the table is not eligible, the launch is too small to fill the machine with runs, or
+    its rows share too few columns for resident strips to pay."""
+    blocks, offsets = layout
+    nnz = blocks.numel() // 2
+    entries = batches * strips_n
+    cus = torch.cuda.get_device_properties(offsets.device).multi_processor_count
+    if nnz * entries < cus * RUN_WALK_PAIRS_MIN:
+        return None
+    generations = max(1, round(nnz * entries / (cus * RUN_WALK_PAIRS)))
+    runs_wanted = max(1, cus * generations // entries)
+    cache = getattr(offsets, "_bsa_runs", None)
+    if cache is None:
+        cache = {}
+        offsets._bsa_runs = cache
+    if runs_wanted not in cache:
+        if torch.cuda.is_current_stream_capturing():
+            return None                     # building synchronises: the first call for a shape runs eagerly
+        target = max(RUN_WALK_PAIRS_MIN, -(-nnz // runs_wanted))
+        for _ in range(4):                  # a cut forced by the strips can leave one run too many: aim higher
+            rs = RunSchedule(blocks, offsets, target, RUN_WALK_STRIPS)
+            if rs.runs <= runs_wanted:
+                break
+            target = -(-target * 11 // 10)
+        cache[runs_wanted] = rs
+    rs = cache[runs_wanted]
+    if rs.runs == 0 or rs.reuse < RUN_WALK_MIN_REUSE:
+        return None
+    rs.waves = max(RUN_WALK_WAVES, -(-rs.strips // 4), -(-rs.pairs // 64))
+    return rs if rs.waves <= 12 else None
 
 
 def _launch(sched, status):
@@ -259,6 +322,17 @@ def sparse_matmul(a, b, mode, row_layout, col_layout, trans_a=False, trans_b=Fal
                 sched.table.data_ptr(), sched.workgroups, sched.waves, crows, ccols, cblocks.numel() // 2, batches,
                 1 if shared else batches, size_n, _k.current_stream()))
         return c
+
+    if (RUN_WALK and mode == "dsd" and not trans_a and not trans_b and a.dtype != torch.float32
+            and size_n % 64 == 0):
+        runs = _run_schedule(layout, batches, size_n // 64)
+        if runs is not None:
+            with torch.cuda.device(a.device):
+                _k.check(_k.lib.bsa_matmul_dsd_runs(
+                    _DTYPES[a.dtype], a.data_ptr(), b.data_ptr(), c.data_ptr(), layout[0].data_ptr(),
+                    layout[1].data_ptr(), runs.table.data_ptr(), runs.runs, runs.strips, runs.pairs, runs.waves,
+                    mask_rows, mask_cols, num_blocks, batches, 1 if shared else batches, size_n, _k.current_stream()))
+            return c
 
     if mode == "sdd":
         sched = schedule_for(layout, SCHEDULE_SDD_F32 if a.dtype == torch.float32 else SCHEDULE_SDD)

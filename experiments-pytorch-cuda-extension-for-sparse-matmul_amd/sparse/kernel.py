@@ -17,6 +17,7 @@ LIBRARY_PATH = os.path.join(_CSRC, "libbsa_hip.so")
 
 BSA_F32, BSA_F16, BSA_BF16 = 0, 1, 2
 BSA_SDD, BSA_DSD, BSA_DDS = 0, 1, 2
+BSA_OK, BSA_ERR_INVALID, BSA_ERR_LAUNCH, BSA_ERR_UNSUPPORTED = 0, -1, -2, -3
 MODES = {"sdd": BSA_SDD, "dsd": BSA_DSD, "dds": BSA_DDS}
 
 _vp, _i, _i64, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
@@ -35,6 +36,9 @@ SIGNATURES = {
     "bsa_matmul_noalloc": (_i, [_i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i,
                                 _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "bsa_matmul_dsd_block64": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "bsa_run_schedule_bytes": (ctypes.c_int64, [_i, _i]),
+    "bsa_run_schedule_build": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, ctypes.c_int64, _vp, _vp]),
+    "bsa_matmul_dsd_runs": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "bsa_softmax_forward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "bsa_softmax_backward": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp]),
     "bsa_to_sparse": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),

@@ -217,6 +217,36 @@ int bsa_matmul_dsd_block64(int dtype, const void *a, const void *b, void *c,
                            int coarse_rows, int coarse_cols, int coarse_nnz, int batches, int sparse_batches,
                            int N, void *stream);
 
+/* ---- DSD over runs of block rows, the dense strips of a run resident in LDS -----
+ * No counterpart in the reference, whose DSD kernel reloads the dense tile of every block
+ * (sparse/native/sparse_smm_gpu.cu:131-155).  c[b] = S(a)[b] * b[b] for the ROW table, no transposes,
+ * fp16 / bf16, N a multiple of 64: the same product, on the same tables, as bsa_matmul(BSA_DSD).
+ * A run is a range of consecutive block rows handled by one workgroup that has a compute unit to
+ * itself: it fetches each distinct 32 x 64 strip of b that its rows name once into LDS (at most 39
+ * strips) and then reads nothing but blocks from memory.  Pays when neighbouring rows share most of
+ * their columns (local + strided / global attention masks); tables with a row of more than
+ * max_strips blocks are not eligible.
+ *   bsa_run_schedule_bytes   device bytes of the schedule of a table
+ *   bsa_run_schedule_build   cuts the rows into runs of about target_pairs pairs (nearest row
+ *                            boundary) and at most max_strips (1..39) distinct columns;
+ *                            counts_out device int32[4]: runs (0: not eligible), strips of the
+ *                            widest run, strips of all runs together (pairs / strips = how often a
+ *                            fetched strip is used), pairs of the longest run
+ *   bsa_matmul_dsd_runs      n_runs, run_strips, run_pairs: counts_out[0], [1], [3]; waves per
+ *                            workgroup (1..12) with run_strips <= 4 waves and run_pairs <= 64 waves.
+ *                            Results agree with bsa_matmul to the rounding of the fp32 sums (the
+ *                            pairs of a row are summed in a different order).
+ */
+int64_t bsa_run_schedule_bytes(int mask_rows, int nnz);
+int bsa_run_schedule_build(const int32_t *row_blocks, const int32_t *row_offsets, int mask_rows, int nnz,
+                           int target_pairs, int max_strips, void *sched, int64_t sched_bytes,
+                           int32_t *counts_out, void *stream);
+int bsa_matmul_dsd_runs(int dtype, const void *a, const void *b, void *c,
+                        const int32_t *row_blocks, const int32_t *row_offsets,
+                        const void *run_sched, int n_runs, int run_strips, int run_pairs, int waves,
+                        int mask_rows, int mask_cols, int nnz, int batches, int sparse_batches,
+                        int N, void *stream);
+
 /* ---- block-sparse softmax ----------------------------------------------
  * Replaces sparse_softmax_forward / sparse_softmax_backward
  * (sparse_softmax.cu:208-258) and their kernels (:113-205), with two additions:
