@@ -147,7 +147,10 @@ __device__ __forceinline__ void stg16_uncounted(void *p, uint4 v)
 }
 
 constexpr int RUN_STRIPS_PER_WAVE = 4;
-constexpr int RUN_DEPTH = 3;      // blocks in flight per wave
+#ifndef BSA_RUN_DEPTH
+#define BSA_RUN_DEPTH 3
+#endif
+constexpr int RUN_DEPTH = BSA_RUN_DEPTH;      // blocks in flight per wave
 
 __device__ __forceinline__ void mailbox_put(const f4v (&acc)[8], float *box)
 {
