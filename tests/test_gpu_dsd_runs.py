@@ -250,3 +250,30 @@ def test_refusals():
     assert K.lib.bsa_run_schedule_build(*args, 8, 8, rs.table.data_ptr(), 16, counts.data_ptr(),
                                         None) == K.BSA_ERR_INVALID              # buffer too small
     assert K.lib.bsa_run_schedule_bytes(rows, L.num_blocks) == RECORD_BYTES * rows + (L.num_blocks + 3) // 4 * 4
+
+
+def test_headline_size_takes_the_run_walk():
+    """4096 tokens, 16 heads, the mask of the benchmark: the launch fills the machine, so ``sparse.matmul`` must walk
+    runs (16 per head: one workgroup per compute unit of a 256-unit GPU), and both walks must agree with the dense
+    fp32 product computed on the GPU; the run walk twice gives the same bits."""
+    import sparse, workloads as wl
+    from sparse import _ops
+    wk = wl.seq4096()
+    L = sparse.SparseLayout(wk["mask"])
+    p, v = (wk["w"].float().abs() * 10).half().cuda(), wk["v"].cuda()
+    rs = _ops._run_schedule(L.row_layout, 16, 1)
+    assert rs is not None and rs.strips <= 32 and rs.reuse > 4
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert rs.runs * 16 <= cus or cus != 256
+    ref = torch.matmul(L.to_dense(p).float(), v.float())
+    out = sparse.matmul(p, v, "dsd", L)
+    assert ((out.float() - ref).abs().max() / ref.abs().max()).item() <= tol_of(torch.float16)
+    row_err = (out.float() - ref).abs().amax(dim=-1) / ref.abs().amax(dim=-1).clamp_min(1e-6)
+    assert row_err.max().item() <= tol_of(torch.float16)
+    assert torch.equal(out, sparse.matmul(p, v, "dsd", L))
+    _ops.RUN_WALK = False
+    try:
+        old = sparse.matmul(p, v, "dsd", L)
+    finally:
+        _ops.RUN_WALK = True
+    assert ((old.float() - out.float()).abs().max() / ref.abs().max()).item() <= tol_of(torch.float16)
