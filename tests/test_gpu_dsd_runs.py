@@ -283,3 +283,41 @@ def test_headline_size_takes_the_run_walk():
     finally:
         _ops.RUN_WALK = True
     assert ((old.float() - out.float()).abs().max() / ref.abs().max()).item() <= tol_of(torch.float16)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_tables_targets_and_waves(seed):
+    """Seeded sweep: masks mixing a local window, strided columns, random blocks and empty rows; any target, strip
+    limit and wave count the entry point accepts.  Every case against the oracle."""
+    import sparse
+    from sparse import kernel as K
+    rng = np.random.RandomState(1000 + seed)
+    rows, cols = int(rng.randint(1, 40)), int(rng.randint(1, 40))
+    i, j = np.indices((rows, cols))
+    mask = np.zeros((rows, cols), dtype=np.int64)
+    if rng.rand() < 0.7:
+        mask |= (np.abs(i - j) < rng.randint(1, 4)).astype(np.int64)
+    if rng.rand() < 0.6:
+        mask |= (j % int(rng.randint(2, 9)) == 0).astype(np.int64)
+    mask |= (rng.rand(rows, cols) < rng.choice([0.0, 0.05, 0.3])).astype(np.int64)
+    if rng.rand() < 0.5:
+        mask &= (j <= i * cols // rows).astype(np.int64)
+    mask[rng.rand(rows) < 0.15] = 0
+    waves = int(rng.randint(1, 13))
+    max_strips = int(rng.randint(1, min(39, 4 * waves) + 1))
+    target = int(rng.choice([1, 3, 8, 20, 64, 200]))
+    width = 64 * int(rng.randint(1, 3))
+    batches = int(rng.choice([1, 2, 9]))
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    rs, _, _ = _build(L, target, max_strips)
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(batches, L.num_blocks, 32, 32, generator=g).half()
+    b = torch.randn(batches, 32 * cols, width, generator=g).half()
+    rc, out = _call(L, rs, a.cuda(), b.cuda(), waves)
+    longest = int(mask.sum(axis=1).max())
+    if longest > max_strips or rs.pairs > 64 * waves:
+        assert (rs.runs == 0) == (longest > max_strips) and rc == K.BSA_ERR_INVALID
+        return
+    assert rc == 0, K.lib.bsa_last_error()
+    assert not torch.isnan(out).any()
+    assert rel_err(to_np(out), mo.matmul(to_np(a), to_np(b), "dsd", mask)) <= tol_of(torch.float16)
