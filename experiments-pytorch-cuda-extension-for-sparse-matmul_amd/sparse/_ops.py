@@ -22,9 +22,9 @@ SOFTMAX_LONGEST_FIRST = True     # long rows are dispatched first: they would ot
 SOFTMAX_WAVES_LONG_ROWS = 8
 SCHEDULE_BLOCK64 = (4, 2, False)        # coarse pairs (64x64 blocks = four tiles) per wavefront; never split
 # DSD on a block=64 layout: True takes the kernel whose wavefronts own whole 64x64 blocks, False walks the layout's
-# 32x32 tiles.  Measured at 4096 tokens, 16 heads, 399 blocks of 64 (bench.py, rows block64_mask_*): 18.8 us against
-# 17.1 us; a wavefront that holds a 64 x 64 fp32 tile needs 227 registers (two waves per SIMD), so the tile walk stays
-# the default.
+# 32x32 tiles.  Measured at 4096 tokens, 16 heads, 399 blocks of 64 (bench.py, rows block64_mask_*): 17.9-18.8 us
+# against 17.1-18.4 us for the group walk over the tiles and 16.5 us for the run walk over them; a wavefront that
+# holds a 64 x 64 fp32 tile needs 227 registers (two waves per SIMD), so the tile walks stay the default.
 USE_BLOCK64_KERNEL = False
 # DSD over a row table with the dense operand stored [K][N]: runs of consecutive block rows whose dense strips stay
 # in LDS (bsa_matmul_dsd_runs), when the table is eligible, a fetched strip serves at least RUN_WALK_MIN_REUSE pairs
