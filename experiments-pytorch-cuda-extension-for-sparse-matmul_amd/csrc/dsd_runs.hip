@@ -208,11 +208,14 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
         wt = wt < e ? wt : last;
         int win_pos, win_byte;
         uint4 blk[RUN_DEPTH][2];
-        auto issue_block = [&](int p, uint4 (&bb)[2]) {             // pair p of a row table names block p
-            const int pc = p < e ? p : last;
-            const half_t *src = spb + (size_t)pc * BS2;
-            bb[0] = ldg16_stream(src);
-            bb[1] = ldg16_stream(src + 16 * BS);
+        // Pair p of a row table names block p.  Past the end of the chunk the request stays (the wait counts the
+        // compiler derives stay exact) but every lane asks for the same 16 bytes of the run's record: one cache line
+        // instead of a block, never used.
+        const half_t *idle = reinterpret_cast<const half_t *>(rec);
+        auto issue_block = [&](int p, uint4 (&bb)[2]) {
+            const half_t *src = spb + (size_t)p * BS2;
+            bb[0] = ldg16_stream(p < e ? src : idle);
+            bb[1] = ldg16_stream(p < e ? src + 16 * BS : idle);
         };
         auto first_requests = [&](auto rounds_c) {
             constexpr int K = decltype(rounds_c)::value;
@@ -295,7 +298,7 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
         int cur = (int)((unsigned)__builtin_amdgcn_readlane(win_pos, 0) >> 16);
         bool first_group = true;
         // one block: its strip out of LDS, eight 16 x 16 x 32 products, then the request for the block
-        // RUN_DEPTH further on (past the chunk's end: its last block again, served by the caches, never used)
+        // RUN_DEPTH further on
         auto step = [&](int p, uint4 (&bb)[2]) {
             if (p < e) {
                 const int gp = (int)((unsigned)__builtin_amdgcn_readlane(win_pos, p - b) >> 16);
