@@ -20,7 +20,8 @@ The K timed steps are run `--repeats` times (default 7); `ms_per_step` / `value`
 runs, the fastest and slowest are reported beside it.  A streaming copy of the softmax's byte count
 (non-temporal 16-byte loads and stores, csrc/bench_yardstick.hip) is timed the same way in the same run:
 `yardstick` says what a plain copy reaches on this box in this minute, and every kernel carries
-`vs_copy` = its algorithmic GB/s over the copy's.
+`vs_copy` = its algorithmic GB/s over the copy's.  The same bytes as a read alone, as a write alone, and a launch
+that moves nothing are timed beside it (`read_us`, `write_us`, `empty_launch_us`).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--sets S] [--no-cpu] [--no-attention] [--no-dense] [--no-configs]
 """
@@ -183,6 +184,29 @@ def main():
     copy_gbs = 2 * copy_bytes / (copy_ms * 1e-3) / 1e9
     yardstick = {"what": "non-temporal copy, 16 B per lane, 4 loads in flight", "bytes_in": copy_bytes, "bytes_out": copy_bytes,
                  "us": round(copy_ms * 1e3, 3), "GBps": round(copy_gbs, 1), "hbm_frac": round(copy_gbs / HBM_PEAK_GBS, 4)}
+    # the same stream as a read alone and as a write alone, and a launch that moves nothing: what the hardware
+    # does with 50 MB in one direction, and what a launch costs before its first byte
+    bench_lib.bsa_bench_read_nt.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    bench_lib.bsa_bench_write_nt.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    bench_lib.bsa_bench_empty.argtypes = [ctypes.c_uint, ctypes.c_void_p]
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def checked(rc):
+        assert rc == 0, rc
+        return sink
+
+    def index_of(w):
+        return next(k for k, v in enumerate(sets) if v is w)
+
+    for key, fn in (("read", lambda w: checked(bench_lib.bsa_bench_read_nt(w["scores"].data_ptr(), sink.data_ptr(), copy_bytes,
+                                                                             torch.cuda.current_stream().cuda_stream))),
+                    ("write", lambda w: checked(bench_lib.bsa_bench_write_nt(copy_dst[index_of(w)].data_ptr(), copy_bytes,
+                                                                               torch.cuda.current_stream().cuda_stream))),
+                    ("empty_launch", lambda w: checked(bench_lib.bsa_bench_empty(2048, torch.cuda.current_stream().cuda_stream)))):
+        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+        yardstick[key + "_us"] = round(ms * 1e3, 3)
+        if key != "empty_launch":
+            yardstick[key + "_GBps"] = round(copy_bytes / (ms * 1e-3) / 1e9, 1)
     del copy_dst
 
     # per-kernel average launch duration: REPS launches per graph, events around the replays
