@@ -321,3 +321,27 @@ def test_random_tables_targets_and_waves(seed):
     assert rc == 0, K.lib.bsa_last_error()
     assert not torch.isnan(out).any()
     assert rel_err(to_np(out), mo.matmul(to_np(a), to_np(b), "dsd", mask)) <= tol_of(torch.float16)
+
+
+def test_run_walk_in_a_hip_graph(small_launches):
+    """The run walk keeps no state and allocates nothing at launch: captured into a HIP graph after one eager call
+    (the schedule is built then), every replay, with other work between the replays, gives the eager result."""
+    import sparse
+    mask = _attention_mask(32, 3, 4)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    g = torch.Generator().manual_seed(21)
+    a = torch.randn(4, L.num_blocks, 32, 32, generator=g).half().cuda()
+    b = torch.randn(4, 32 * 32, 64, generator=g).half().cuda()
+    eager = sparse.matmul(a, b, "dsd", L)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            out = sparse.matmul(a, b, "dsd", L)
+    for r in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), r
+        eager = sparse.matmul(a, b, "dsd", L)          # eager work between the replays
