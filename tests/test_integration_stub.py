@@ -1,4 +1,4 @@
-"""The reference-side binding shown in INTEGRATION.md ("Option B"): the code block a maintainer of the
+"""The reference-side binding of the integration notes ("Option B"): the code block a maintainer of the
 reference would paste as sparse/kernel.py is taken out of the document and executed as it stands.
 
 Without a GPU: it loads the library and its ctypes signatures agree with the bindings of this package.
@@ -26,7 +26,7 @@ def _stub_namespace():
     code = re.search(r"```python\n(.*?)```", section, re.S).group(1)
     assert '"libbsa_hip.so"' in code
     ns = {}
-    exec(compile(code.replace('"libbsa_hip.so"', repr(k.LIBRARY_PATH)), "INTEGRATION.md:Option B", "exec"), ns)
+    exec(compile(code.replace('"libbsa_hip.so"', repr(k.LIBRARY_PATH)), "<Option B stub>", "exec"), ns)
     return ns
 
 
