@@ -393,6 +393,24 @@ def main():
             ops64.USE_BLOCK64_KERNEL = False
         configs["block64_mask_tiles"] = l64.num_blocks
         del sets64
+
+        # The headline products in fp32 (v_mfma_f32_32x32x2_f32: 157 TFLOP/s bounds them before HBM does), on
+        # rotating operand sets (three: an fp32 set is twice the bytes).
+        sets32 = [{k: w[k].float() for k in ("q", "k", "v", "scores", "w")} for w in sets[:3]]
+        turn32 = [0]
+
+        def next32():
+            turn32[0] += 1
+            return sets32[turn32[0] % len(sets32)]
+
+        b32 = (nnz * 1024 + 2 * seq * D) * B * 4
+        for name, fn in (("sdd", lambda: (lambda w: sparse.matmul(w["q"], w["k"], "sdd", layout, False, True))(next32())),
+                         ("dsd", lambda: (lambda w: sparse.matmul(w["scores"], w["v"], "dsd", layout))(next32())),
+                         ("dds", lambda: (lambda w: sparse.matmul(w["v"], w["w"], "dds", layout, True, False))(next32()))):
+            run_config(f"seq4096_{name}_fp32", fn, 2 * len(sets32), flops=flops_one, nbytes=b32)
+            configs[f"seq4096_{name}_fp32"]["mfma_f32_frac"] = round(
+                configs[f"seq4096_{name}_fp32"]["nnz_TFLOPs"] / 157.3, 4)
+        del sets32
         c5 = on_gpu(wl.config5())
         l5 = sparse.SparseLayout(c5["mask"])
         n5, b5 = l5.num_blocks, 48

@@ -4,14 +4,16 @@
 // unfinished fp16 twin sparse/native/sparse_hmm_gpu.cu:26-317.  Nothing of
 // their structure is kept: every nonzero 32x32 block is one MFMA tile owned by
 // ONE wavefront (v_mfma_f32_32x32x16_f16, fp32 accumulate; v_mfma_f32_32x32x2_f32
-// for fp32).  fp16 tiles are fetched with fully coalesced requests (lane l takes
-// 16-byte pieces l and l + 64 of a 2 KB tile, whatever its orientation), parked
-// in a wave-private, XOR-swizzled LDS tile and read back in MFMA layout:
-// ds_read_b128 when the contraction index is contiguous in the tile,
-// ds_read_b64_tr_b16 (hardware transpose) when it is the slow index.  MFMA-layout
-// loads straight from global memory (lane = row, 16 bytes at row stride) were
-// measured at a third of the coalesced rate and are only used by the fp32
-// kernels.  Data touched once (sparse blocks, results) moves with non-temporal
+// for fp32).  Tiles are fetched with fully coalesced requests (lane l takes
+// 16-byte pieces l and l + 64 of a 2 KB fp16 tile, whatever its orientation; a
+// request of an fp32 tile covers 8 whole 128-byte rows), parked in a wave-private
+// LDS tile (XOR-swizzled for fp16, padded rows for fp32) and read back in MFMA
+// layout: ds_read_b128 when the contraction index is contiguous in the tile,
+// ds_read_b64_tr_b16 (hardware transpose; ds_read_b32 for fp32) when it is the
+// slow index.  MFMA-layout loads straight from global memory (lane = row, 16
+// bytes at row stride) were measured at a third of the coalesced rate; only the
+// fp32 fallbacks (K > 128, a dense dimension that is no multiple of 64) keep
+// them.  Data touched once (sparse blocks, results) moves with non-temporal
 // loads and stores; dense tiles, which are re-read out of L2, do not.  No
 // workgroup barrier sits in any inner loop, and no load under a condition sits
 // in the steady state of a block loop (tails are peeled): behind a conditional
@@ -196,7 +198,8 @@ __global__ __launch_bounds__(512) void sdd_f16_kernel(
 
 // ---------------------------------------------------------------------------
 // fp32 operand tiles: 16 floats per lane, k = 16 * (lane / 32) + 0..15 of one
-// index.  Both memory orientations load straight into registers.
+// index.  Both memory orientations load straight into registers (the fallback
+// kernels sdd_f32_kernel and gw_f32_kernel; the tiled kernels below stage through LDS).
 // ---------------------------------------------------------------------------
 template <bool KC, bool PERMUTED>
 __device__ __forceinline__ void ldg_tile_f32(const float *src, size_t ld, float (&v)[16])
@@ -268,6 +271,142 @@ __global__ __launch_bounds__(512) void sdd_f32_kernel(
             }
         }
         store16_f32(cb + (size_t)d.idx * BS2 + (l & 31) * BS + 16 * (l >> 5), acc);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// fp32 operand tiles through LDS.  A 32 x 32 fp32 tile (rows 128 bytes) is fetched with four fully
+// coalesced requests (a request covers 8 whole rows) and parked in a wave-private LDS tile in its memory
+// orientation, rows 36 floats apart and rows 16-31 another 32 floats on.  The MFMA operand (16 floats per
+// lane: one index, k = 16 (lane / 32) .. + 15) is read back with four ds_read_b128 when k is the
+// contiguous index (a 16-lane phase reads 16 rows whose offsets 36 r + 32 [r >= 16] fall into 16 different
+// groups of four banks, for the natural and for the perm16 row order) and with sixteen ds_read_b32 when k
+// is the row (lanes of the lower half read banks b .. b + 31 of row k, the upper half the same banks + 32
+// of row k + 16: that is what the extra 32 floats are for).
+// ---------------------------------------------------------------------------
+constexpr int F32_TILE_BYTES = 4864;     // 32 * 36 + 32 floats, rounded up to 128 bytes
+__device__ __forceinline__ int f32_tile_off(int row, int col) { return row * 36 + ((row >> 4) << 5) + col; }
+
+template <bool STREAM>
+__device__ __forceinline__ void ldg_tile32_f32(const float *src, size_t ld, uint4 (&raw)[4])
+{
+    const int l = lane_id();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float *p = src + (size_t)((l >> 3) + 8 * j) * ld + 4 * (l & 7);
+        raw[j] = STREAM ? ldg16_stream(p) : ldg16(p);
+    }
+}
+
+__device__ __forceinline__ void lds_put_f32(float *tile, const uint4 (&raw)[4])
+{
+    const int l = lane_id();
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<uint4 *>(tile + f32_tile_off((l >> 3) + 8 * j, 4 * (l & 7))) = raw[j];
+}
+
+template <bool KC, bool PERMUTED>
+__device__ __forceinline__ void lds_get_f32(const float *tile, float (&v)[16])
+{
+    const int l = lane_id();
+    const int i = PERMUTED ? perm16(l & 31) : (l & 31);
+    const int k0 = 16 * (l >> 5);
+    if (KC) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 x = *reinterpret_cast<const float4 *>(tile + f32_tile_off(i, k0 + 4 * q));
+            v[4 * q] = x.x; v[4 * q + 1] = x.y; v[4 * q + 2] = x.z; v[4 * q + 3] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 16; ++t) v[t] = tile[f32_tile_off(k0 + t, i)];
+    }
+}
+
+// SDD fp32 with K = 32 KBT <= 128: the operands of the wave's block row stay in registers (16 KBT floats per
+// lane), the tiles of block p + 1 are requested as soon as those of block p have left their registers for LDS,
+// and the products of block p run while they arrive.
+template <bool A_KC, bool B_KC, int KBT>
+__global__ __launch_bounds__(512) void sdd_f32_tiled_kernel(
+    const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ c,
+    const BlockDesc *__restrict__ blocks, const SchedEntry *__restrict__ sched,
+    int n_swg, int batches, int nnz, int M, int N, int K)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    if (e.group < 0 || e.begin >= e.end) return;
+    float *tiles = reinterpret_cast<float *>(lds_raw + (size_t)w * KBT * F32_TILE_BYTES);
+    const float *ab = a + (size_t)batch * M * K;
+    const float *bb = b + (size_t)batch * N * K;
+    float *cb = c + (size_t)batch * nnz * BS2;
+    const int r = e.group;
+
+    uint4 raw[KBT][4];
+    float aop[KBT][16];
+    DescWindow win;
+    const int first_end = e.begin + WAVE < e.end ? e.begin + WAVE : e.end;
+    win.fetch(blocks, e.begin, first_end);
+#pragma unroll
+    for (int kb = 0; kb < KBT; ++kb) {
+        if (A_KC) ldg_tile32_f32<false>(ab + (size_t)(BS * r) * K + BS * kb, K, raw[kb]);
+        else ldg_tile32_f32<false>(ab + (size_t)(BS * kb) * M + BS * r, M, raw[kb]);
+    }
+    auto request = [&](int p) {
+        const int cblk = win.get(p).col();
+#pragma unroll
+        for (int kb = 0; kb < KBT; ++kb) {
+            if (B_KC) ldg_tile32_f32<false>(bb + (size_t)(BS * cblk) * K + BS * kb, K, raw[kb]);
+            else ldg_tile32_f32<false>(bb + (size_t)(BS * kb) * N + BS * cblk, N, raw[kb]);
+        }
+    };
+    auto park = [&]() {
+        wave_lds_fence();
+#pragma unroll
+        for (int kb = 0; kb < KBT; ++kb) lds_put_f32(tiles + kb * (F32_TILE_BYTES / 4), raw[kb]);
+        wave_lds_fence();
+    };
+    auto multiply = [&](int p) {
+        f16v acc = {0};
+#pragma unroll
+        for (int kb = 0; kb < KBT; ++kb) {
+            float bop[16];
+            lds_get_f32<B_KC, true>(tiles + kb * (F32_TILE_BYTES / 4), bop);
+#pragma unroll
+            for (int t = 0; t < 16; ++t) acc = mfma_f32(bop[t], aop[kb][t], acc);
+        }
+        // a lane holds 16 consecutive columns of one row; the block leaves through LDS as four whole
+        // kilobytes (64-byte pieces at 128-byte stride straight from the registers write at a third of the rate)
+        wave_lds_fence();
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<float4 *>(tiles + f32_tile_off(l & 31, 16 * (l >> 5) + 4 * q)) =
+                make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+        wave_lds_fence();
+        float *dst = cb + (size_t)win.get(p).idx * BS2;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            stg16_stream(dst + 4 * (l + 64 * j),
+                         *reinterpret_cast<const uint4 *>(tiles + f32_tile_off((l >> 3) + 8 * j, 4 * (l & 7))));
+    };
+    park();
+#pragma unroll
+    for (int kb = 0; kb < KBT; ++kb) lds_get_f32<A_KC, false>(tiles + kb * (F32_TILE_BYTES / 4), aop[kb]);
+    for (int seg = e.begin; seg < e.end; seg += WAVE) {
+        const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+        if (seg != e.begin) win.fetch(blocks, seg, seg_end);
+        request(seg);
+        for (int p = seg; p + 1 < seg_end; ++p) {
+            park();
+            request(p + 1);
+            multiply(p);
+        }
+        park();
+        multiply(seg_end - 1);
     }
 }
 
@@ -853,6 +992,91 @@ __global__ __launch_bounds__(512) void gw_f32_kernel(
     }
 }
 
+// The same walk for a dense dimension that is a multiple of 64, with every operand tile fetched by coalesced
+// requests and turned into MFMA operands through the wave's LDS tile (one tile at a time: the partial-tile
+// area of the team reduce is enough), and with the three tiles of pair p + 1 requested before the 32 products
+// of pair p are issued.
+template <bool S_KC, bool D_KC, bool DSD>
+__global__ __launch_bounds__(512) void gw_f32_tiled_kernel(
+    const float *__restrict__ sp, const float *__restrict__ dn, float *__restrict__ out,
+    const BlockDesc *__restrict__ blocks, const SchedGroup *__restrict__ sched_groups,
+    const SchedEntry *__restrict__ sched, SplitWorkspace ws,
+    int n_swg, int batches, int nnz, int DN, int KT, int XT, int sp_shared)
+{
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    static_assert(F32_TILE_BYTES <= GW_LDS_PER_WAVE, "the operand tile shares the wave's reduce area");
+    int batch, swg;
+    if (!map_workgroup(n_swg, batches, batch, swg)) return;
+    const int w = wave_id(), l = lane_id();
+    const int W = (int)(blockDim.x >> 6);
+    const SchedEntry e = sched[swg * W + w];
+    const int y0 = 64 * (int)blockIdx.y;
+    const float *spb = sp + (sp_shared ? 0 : (size_t)batch * nnz * BS2);
+    const float *dnb = dn + (size_t)batch * DN * KT;
+    float *tile = reinterpret_cast<float *>(lds_raw + (size_t)w * GW_LDS_PER_WAVE);
+
+    f16v acc[2] = {{0}, {0}};
+    if (e.group >= 0) {
+        DescWindow win;
+        uint4 sraw[4], draw[2][4];
+        auto request = [&](int p) {
+            const BlockDesc d = win.get(p);
+            const int kblk = S_KC ? d.col() : d.row();
+            ldg_tile32_f32<true>(spb + (size_t)d.idx * BS2, BS, sraw);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (D_KC) ldg_tile32_f32<false>(dnb + (size_t)(y0 + 32 * t) * KT + BS * kblk, KT, draw[t]);
+                else ldg_tile32_f32<false>(dnb + (size_t)(BS * kblk) * DN + y0 + 32 * t, DN, draw[t]);
+            }
+        };
+        auto operands = [&](float (&sv)[16], float (&dv)[2][16]) {
+            wave_lds_fence();
+            lds_put_f32(tile, sraw);
+            wave_lds_fence();
+            lds_get_f32<S_KC, !DSD>(tile, sv);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                wave_lds_fence();
+                lds_put_f32(tile, draw[t]);
+                wave_lds_fence();
+                lds_get_f32<D_KC, DSD>(tile, dv[t]);
+            }
+        };
+        auto multiply = [&](const float (&sv)[16], const float (&dv)[2][16]) {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                if (DSD) {
+                    acc[0] = mfma_f32(dv[0][k], sv[k], acc[0]);
+                    acc[1] = mfma_f32(dv[1][k], sv[k], acc[1]);
+                } else {
+                    acc[0] = mfma_f32(sv[k], dv[0][k], acc[0]);
+                    acc[1] = mfma_f32(sv[k], dv[1][k], acc[1]);
+                }
+            }
+        };
+        for (int seg = e.begin; seg < e.end; seg += WAVE) {
+            const int seg_end = seg + WAVE < e.end ? seg + WAVE : e.end;
+            win.fetch(blocks, seg, seg_end);
+            request(seg);
+            float sv[16], dv[2][16];
+            for (int p = seg; p + 1 < seg_end; ++p) {
+                operands(sv, dv);
+                request(p + 1);
+                multiply(sv, dv);
+            }
+            operands(sv, dv);
+            multiply(sv, dv);
+        }
+        wave_lds_fence();    // the tile area becomes the wave's partial tile below
+    }
+    if (team_reduce<f16v, 2, 16>(acc, e, w, lds_raw) &&
+        (e.parts() <= 1 || split_combine<f16v, 2, 16>(acc, e, sched_groups[e.group], ws, batch))) {
+        float *ob = out + (size_t)batch * XT * DN;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) store16_f32(ob + gw_out_offset<DSD>(e.group, y0, t, l, DN, XT), acc[t]);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
@@ -882,9 +1106,20 @@ template <bool A_KC, bool B_KC>
 static hipError_t launch_sdd_f32(const MatmulArgs &p, hipStream_t st)
 {
     dim3 grid(grid_x(p.sched_wgs, p.batches)), block(64 * p.sched_waves);
-    sdd_f32_kernel<A_KC, B_KC><<<grid, block, 0, st>>>(
-        (const float *)p.a, (const float *)p.b, (float *)p.c, (const BlockDesc *)p.blocks,
-        sched_slots(p), p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K);
+#define BSA_SDD_ARGS (const float *)p.a, (const float *)p.b, (float *)p.c, (const BlockDesc *)p.blocks, \
+                     sched_slots(p), p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K
+    const int kbs = p.K / BS;
+    const size_t lds = (size_t)p.sched_waves * kbs * F32_TILE_BYTES;
+    if (kbs <= 4 && lds <= 65536) {
+        switch (kbs) {
+            case 1: sdd_f32_tiled_kernel<A_KC, B_KC, 1><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+            case 2: sdd_f32_tiled_kernel<A_KC, B_KC, 2><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+            case 3: sdd_f32_tiled_kernel<A_KC, B_KC, 3><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+            default: sdd_f32_tiled_kernel<A_KC, B_KC, 4><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+        }
+    } else
+        sdd_f32_kernel<A_KC, B_KC><<<grid, block, 0, st>>>(BSA_SDD_ARGS);
+#undef BSA_SDD_ARGS
     return hipGetLastError();
 }
 
@@ -937,9 +1172,13 @@ static hipError_t launch_gw_t(int dtype, const void *sp, const void *dn, const M
         else gw_f16_kernel<S_KC, D_KC, DSD, GW_PREFETCH_DEPTH, true, false><<<grid, block, lds, st>>>(BSA_GW_ARGS);
     } else
 #undef BSA_GW_ARGS
-        gw_f32_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(
-            (const float *)sp, (const float *)dn, (float *)p.c, (const BlockDesc *)p.blocks,
-            sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0);
+    {
+#define BSA_GW32_ARGS (const float *)sp, (const float *)dn, (float *)p.c, (const BlockDesc *)p.blocks, \
+                      sched_groups(p), sched_slots(p), ws, p.sched_wgs, p.batches, p.nnz, DN, KT, XT, p.sparse_shared ? 1 : 0
+        if (full) gw_f32_tiled_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(BSA_GW32_ARGS);
+        else gw_f32_kernel<S_KC, D_KC, DSD><<<grid, block, lds, st>>>(BSA_GW32_ARGS);
+#undef BSA_GW32_ARGS
+    }
     return hipGetLastError();
 }
 
