@@ -22,6 +22,9 @@ extern "C" int bsa_lds_access(const char *name, int permuted, int arg0, int arg1
         else if (!strcmp(name, "get_strip16")) a = get_strip16_addr(lane, arg0, arg1);
         else if (!strcmp(name, "put_result")) a = put_result_addr(lane, arg0);
         else if (!strcmp(name, "get_linear")) a = get_linear_addr(lane, arg0);
+        else if (!strcmp(name, "put_f32")) a = put_f32_addr(lane, arg0);
+        else if (!strcmp(name, "get_f32_kc")) a = get_f32_kc_addr(permuted, lane, arg0);
+        else if (!strcmp(name, "get_f32_ks")) a = get_f32_ks_addr(permuted, lane, arg0);
         else return -1;
         addr64[lane] = a;
     }

@@ -143,4 +143,32 @@ BSA_HD constexpr int get_linear_addr(int lane, int q)
     return 16 * kc_slot(c >> 2, c & 3);
 }
 
+// ---- fp32 tiles (32 x 32 floats = 4 KB, stored in their memory orientation) ---------------------
+// Row r of the tile starts 36 r floats into the LDS tile, rows 16-31 another 32 floats on.  A 16-lane
+// phase of a 16-byte access that takes the same columns of 16 different rows then touches 16 different
+// groups of four banks (9 r + 8 [r >= 16] mod 16 runs through all of them for r = 0..15, for 16..31 and
+// for both halves of the perm16 order), and a 4-byte access of 32 consecutive columns of row k by the
+// lower lane half and of row k + 16 by the upper half covers all 64 banks once.  The linear access
+// (put_f32_addr: a phase takes the 8 pieces of two NEIGHBOURING rows, whose 32-float windows are 36
+// floats apart) meets in 4 of the 64 banks: two clocks per phase instead of one.  Phases that take rows
+// 16 apart are conflict-free, but their requests cover a stored block in two runs of 512 bytes instead
+// of one kilobyte, and the group walks measured 2-4 us slower with them at 4096 tokens, 16 heads.
+constexpr int F32_TILE_FLOATS = 32 * 36 + 32;
+BSA_HD constexpr int f32_tile_off(int row, int col) { return row * 36 + ((row >> 4) << 5) + col; }
+// registers <-> LDS in memory order, 16 bytes per lane: request j of lane l moves piece
+// (row l / 8 + 8 j, columns 4 (l % 8) .. + 3); the 64 lanes of a request cover 8 whole consecutive rows
+BSA_HD constexpr int put_f32_addr(int lane, int j) { return 4 * f32_tile_off((lane >> 3) + 8 * j, 4 * (lane & 7)); }
+// LDS -> MFMA operand (v_mfma_f32_32x32x2_f32: lane = index, k = 16 (lane / 32) + 0..15), tile stored
+// [index][k]: 16-byte read q gives k = 16 h + 4 q .. + 3.  The SDD result (lane = row, 16 consecutive
+// columns 16 h ..) is parked with the same addresses.
+BSA_HD constexpr int get_f32_kc_addr(bool permuted, int lane, int q)
+{
+    return 4 * f32_tile_off(permuted ? perm16(lane & 31) : (lane & 31), 16 * (lane >> 5) + 4 * q);
+}
+// tile stored [k][index]: 4-byte read t gives k = 16 h + t
+BSA_HD constexpr int get_f32_ks_addr(bool permuted, int lane, int t)
+{
+    return 4 * f32_tile_off(16 * (lane >> 5) + t, permuted ? perm16(lane & 31) : (lane & 31));
+}
+
 }  // namespace bsa

@@ -277,16 +277,13 @@ __global__ __launch_bounds__(512) void sdd_f32_kernel(
 // ---------------------------------------------------------------------------
 // fp32 operand tiles through LDS.  A 32 x 32 fp32 tile (rows 128 bytes) is fetched with four fully
 // coalesced requests (a request covers 8 whole rows) and parked in a wave-private LDS tile in its memory
-// orientation, rows 36 floats apart and rows 16-31 another 32 floats on.  The MFMA operand (16 floats per
-// lane: one index, k = 16 (lane / 32) .. + 15) is read back with four ds_read_b128 when k is the
-// contiguous index (a 16-lane phase reads 16 rows whose offsets 36 r + 32 [r >= 16] fall into 16 different
-// groups of four banks, for the natural and for the perm16 row order) and with sixteen ds_read_b32 when k
-// is the row (lanes of the lower half read banks b .. b + 31 of row k, the upper half the same banks + 32
-// of row k + 16: that is what the extra 32 floats are for).
+// orientation, rows padded: the address maps put_f32_addr / get_f32_kc_addr / get_f32_ks_addr of
+// lds_index_math.hpp (byte addresses; the bank-model tests replay them).  The MFMA
+// operand (16 floats per lane: one index, k = 16 (lane / 32) .. + 15) is read back with four
+// ds_read_b128 when k is the contiguous index and with sixteen ds_read_b32 when k is the row.
 // ---------------------------------------------------------------------------
-constexpr int F32_TILE_BYTES = 4864;     // 32 * 36 + 32 floats, rounded up to 128 bytes
-__device__ __forceinline__ int f32_tile_off(int row, int col) { return row * 36 + ((row >> 4) << 5) + col; }
-
+constexpr int F32_TILE_BYTES = 4864;     // F32_TILE_FLOATS floats, rounded up to 128 bytes
+static_assert(4 * F32_TILE_FLOATS <= F32_TILE_BYTES, "fp32 tile size");
 template <bool STREAM>
 __device__ __forceinline__ void ldg_tile32_f32(const float *src, size_t ld, uint4 (&raw)[4])
 {
@@ -303,24 +300,22 @@ __device__ __forceinline__ void lds_put_f32(float *tile, const uint4 (&raw)[4])
     const int l = lane_id();
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-        *reinterpret_cast<uint4 *>(tile + f32_tile_off((l >> 3) + 8 * j, 4 * (l & 7))) = raw[j];
+        *reinterpret_cast<uint4 *>(tile + put_f32_addr(l, j) / 4) = raw[j];
 }
 
 template <bool KC, bool PERMUTED>
 __device__ __forceinline__ void lds_get_f32(const float *tile, float (&v)[16])
 {
     const int l = lane_id();
-    const int i = PERMUTED ? perm16(l & 31) : (l & 31);
-    const int k0 = 16 * (l >> 5);
     if (KC) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const float4 x = *reinterpret_cast<const float4 *>(tile + f32_tile_off(i, k0 + 4 * q));
+            const float4 x = *reinterpret_cast<const float4 *>(tile + get_f32_kc_addr(PERMUTED, l, q) / 4);
             v[4 * q] = x.x; v[4 * q + 1] = x.y; v[4 * q + 2] = x.z; v[4 * q + 3] = x.w;
         }
     } else {
 #pragma unroll
-        for (int t = 0; t < 16; ++t) v[t] = tile[f32_tile_off(k0 + t, i)];
+        for (int t = 0; t < 16; ++t) v[t] = tile[get_f32_ks_addr(PERMUTED, l, t) / 4];
     }
 }
 
@@ -384,14 +379,14 @@ __global__ __launch_bounds__(512) void sdd_f32_tiled_kernel(
         wave_lds_fence();
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            *reinterpret_cast<float4 *>(tiles + f32_tile_off(l & 31, 16 * (l >> 5) + 4 * q)) =
+            *reinterpret_cast<float4 *>(tiles + get_f32_kc_addr(false, l, q) / 4) =
                 make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
         wave_lds_fence();
         float *dst = cb + (size_t)win.get(p).idx * BS2;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             stg16_stream(dst + 4 * (l + 64 * j),
-                         *reinterpret_cast<const uint4 *>(tiles + f32_tile_off((l >> 3) + 8 * j, 4 * (l & 7))));
+                         *reinterpret_cast<const uint4 *>(tiles + put_f32_addr(l, j) / 4));
     };
     park();
 #pragma unroll

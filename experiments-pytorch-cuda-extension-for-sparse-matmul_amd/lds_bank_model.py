@@ -102,12 +102,22 @@ KERNEL_ACCESSES = [
     ("get_strip16", 8, [dict(arg0=t, arg1=h) for t in range(4) for h in (0, 1)]),
     ("put_result", 16, [dict(arg0=j) for j in (0, 1)]),
     ("get_linear", 16, [dict(arg0=q) for q in (0, 1)]),
+    # fp32 tiles: written and read back linearly (put_f32: both directions), read as MFMA operands along k
+    # (get_f32_kc: also the write of the SDD result) and across k (get_f32_ks)
+    ("put_f32", 16, [dict(arg0=j) for j in range(4)]),
+    ("get_f32_kc", 16, [dict(permuted=p, arg0=q) for p in (False, True) for q in range(4)]),
+    ("get_f32_ks", 4, [dict(permuted=p, arg0=t) for p in (False, True) for t in range(16)]),
 ]
 
 
+# Accesses that are NOT conflict-free by design, with the clocks the model must find over the ideal: the linear
+# access of an fp32 tile takes the 8 pieces of two neighbouring rows per phase, whose windows share 4 of the 64
+# banks (csrc/lds_index_math.hpp says why that mapping is kept).
+KNOWN_COST_FACTOR = {"put_f32": 2}
+
 # how the probe binary (csrc/lds_bank_probe.hip) issues each access
 PROBE_OPS = {"put_kc": "w128", "put_ks": "w128", "put_strip": "w128", "put_strip_swapped": "w128", "put_result": "w128", "put_strip16": "w128", "get_strip16": "tr64",
-             "get_kc": "b128", "get_linear": "b128", "get_ks": "tr64", "get_strip": "tr64", "get_kc_tr_swapped": "tr64"}
+             "get_kc": "b128", "get_linear": "b128", "put_f32": "w128", "get_f32_kc": "b128", "get_f32_ks": "b32", "get_ks": "tr64", "get_strip": "tr64", "get_kc_tr_swapped": "tr64"}
 
 
 def _probe(binary: str, op: str, addresses: Sequence[int]) -> float:
