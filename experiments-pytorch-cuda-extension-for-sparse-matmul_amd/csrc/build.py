@@ -9,7 +9,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["api.hip", "layout_build.hip", "matmul.hip", "dsd_runs.hip", "softmax.hip", "attention.hip", "block_copy.hip"]
-HEADERS = ["bench_yardstick.hip", "bsa_device.hpp", "lds_tiles.hpp", "lds_index_math.hpp", "bsa_internal.hpp", os.path.join("..", "..", "include", "bsa.h")]
+HEADERS = ["bench_yardstick.hip", "bsa_device.hpp", "lds_tiles.hpp", "lds_index_math.hpp", "bsa_internal.hpp", "group_walk.hpp", os.path.join("..", "..", "include", "bsa.h")]
 LIB = os.path.join(HERE, "libbsa_hip.so")
 
 FLAGS = [

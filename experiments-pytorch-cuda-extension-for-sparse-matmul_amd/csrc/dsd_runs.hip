@@ -22,6 +22,7 @@
 #include "bsa_device.hpp"
 #include "bsa_internal.hpp"
 #include "lds_tiles.hpp"
+#include "group_walk.hpp"
 
 namespace bsa {
 
@@ -126,26 +127,6 @@ hipError_t launch_run_schedule_build(const int32_t *row_blocks, const int32_t *r
 }
 
 // ---- the walk ---------------------------------------------------------------------------------------
-// workgroup barrier that orders LDS traffic only: global loads in flight stay in flight
-__device__ __forceinline__ void lds_barrier()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-// A 16-byte store the compiler does not see as a memory instruction, for the store of a finished row
-// between two blocks of the pipelined walk: behind a store under a condition the compiler would wait for
-// every load in flight, which cancels the prefetch.  The hardware reads the data registers when the
-// store issues and a wave does not end before its stores are acknowledged; the one rule the compiler
-// would otherwise keep for us is that a store of more than 8 bytes is followed by wait states before its
-// data registers are overwritten (s_nop).
-__device__ __forceinline__ void stg16_uncounted(void *p, uint4 v)
-{
-    u32x4 w = {v.x, v.y, v.z, v.w};
-    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 2" ::"v"(p), "v"(w) : "memory");
-}
-
 constexpr int RUN_STRIPS_PER_WAVE = 4;
 #ifndef BSA_RUN_DEPTH
 #define BSA_RUN_DEPTH 3

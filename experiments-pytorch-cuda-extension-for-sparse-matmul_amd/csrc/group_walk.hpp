@@ -1,0 +1,96 @@
+// Pieces the walks over groups of a block table share (matmul.hip, bin_walk.hip): where a wave's
+// 32 x 64 result tile goes, and how the parts of a group that was cut across workgroups meet.
+#pragma once
+
+#include "bsa_device.hpp"
+
+namespace bsa {
+
+constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + 4 KB), reused for the fp32 partial tile
+
+// workgroup barrier that orders LDS traffic only: global loads in flight stay in flight
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// A 16-byte store the compiler does not see as a memory instruction, for the store of a finished group
+// between two blocks of a pipelined walk: behind a store under a condition the compiler would wait for
+// every load in flight, which cancels the prefetch.  The hardware reads the data registers when the
+// store issues and a wave does not end before its stores are acknowledged; a wave's memory instructions
+// retire in order, so a store the compiler did not count only makes its later waits stricter.  Two rules
+// the compiler would otherwise keep for us: a store of more than 8 bytes is followed by wait states
+// before its data registers are overwritten (the s_nop), and the data and address registers must be
+// results of VALU instructions (conversions, address arithmetic), never of an MFMA directly: a register
+// written by the matrix core needs wait states before a memory instruction reads it that nobody inserts
+// here.  -DBSA_PLAIN_STORES builds the walks with ordinary stores instead (same results).
+__device__ __forceinline__ void stg16_uncounted(void *p, uint4 v)
+{
+#ifdef BSA_PLAIN_STORES
+    *reinterpret_cast<uint4 *>(p) = v;
+#else
+    u32x4 w = {v.x, v.y, v.z, v.w};
+    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 2" ::"v"(p), "v"(w) : "memory");
+#endif
+}
+
+template <bool DSD>
+__device__ __forceinline__ size_t gw_out_offset(int g, int y0, int yt, int l, int DN, int XT)
+{
+    int h = l >> 5, i = l & 31;
+    if (DSD) return (size_t)(BS * g + i) * DN + y0 + 32 * yt + 16 * h;
+    return (size_t)(y0 + 32 * yt + i) * XT + BS * g + 16 * h;
+}
+
+// Split groups: every part parks its fp32 partial tile in the workspace and bumps
+// the group's counter; the part that arrives last adds the tiles up in part order
+// (so the sum does not depend on arrival order), resets the counter and returns
+// true: it stores the result.  Publication follows the release / acquire pattern
+// of split_publish / split_consume (bsa_device.hpp).
+struct SplitWorkspace {
+    int *counters;     // [batches][strips][split_groups], zero between launches
+    float *tiles;      // [batches][strips][tile_slots][2048]
+    int tile_slots, split_groups;
+};
+
+// part `part` of `parts`; the group's tiles start at `tile_slot`, its counter is number `counter_index`
+template <class V, int NT, int EV>
+__device__ __forceinline__ bool split_combine_at(V (&acc)[NT], int part, int parts, int tile_slot, int counter_index,
+                                                 const SplitWorkspace &ws, int batch)
+{
+    const int l = lane_id();
+    const size_t cell = (size_t)batch * gridDim.y + blockIdx.y;
+    float *tile0 = ws.tiles + (cell * ws.tile_slots + tile_slot) * 2048;
+    float *mine = tile0 + (size_t)part * 2048;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < EV; ++v) park_store(mine + (t * EV + v) * WAVE + l, acc[t][v]);
+    int *counter = ws.counters + cell * ws.split_groups + counter_index;
+    if (split_publish(counter) != parts - 1) return false;
+    split_consume();
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < EV; ++v) acc[t][v] = 0.f;
+    for (int p = 0; p < parts; ++p) {
+        const float *src = tile0 + (size_t)p * 2048;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int v = 0; v < EV; ++v) acc[t][v] += park_load(src + (t * EV + v) * WAVE + l);
+    }
+    split_reset(counter);
+    return true;
+}
+
+template <class V, int NT, int EV>
+__device__ __forceinline__ bool split_combine(V (&acc)[NT], const SchedEntry &e, const SchedGroup &sg,
+                                              const SplitWorkspace &ws, int batch)
+{
+    return split_combine_at<V, NT, EV>(acc, e.part(), e.parts(), sg.tile_slot, sg.split_index, ws, batch);
+}
+
+}  // namespace bsa

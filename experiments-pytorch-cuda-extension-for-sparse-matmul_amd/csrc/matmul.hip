@@ -34,11 +34,11 @@
 #include "bsa_device.hpp"
 #include "lds_tiles.hpp"
 #include "bsa_internal.hpp"
+#include "group_walk.hpp"
 #include "../../include/bsa.h"
 
 namespace bsa {
 
-constexpr int GW_LDS_PER_WAVE = 8192;   // staging tiles (2 KB + 4 KB), reused for the fp32 partial tile
 #ifndef BSA_GW_DEPTH
 #define BSA_GW_DEPTH 2
 #endif
@@ -418,14 +418,6 @@ __global__ __launch_bounds__(512) void sdd_f32_tiled_kernel(
 //   D_KC  the dense operand is stored [DN][KT]; otherwise [KT][DN]
 //   DSD   output is [XT][DN] (y contiguous); otherwise (DDS) [DN][XT]
 // ---------------------------------------------------------------------------
-template <bool DSD>
-__device__ __forceinline__ size_t gw_out_offset(int g, int y0, int yt, int l, int DN, int XT)
-{
-    int h = l >> 5, i = l & 31;
-    if (DSD) return (size_t)(BS * g + i) * DN + y0 + 32 * yt + 16 * h;
-    return (size_t)(y0 + 32 * yt + i) * XT + BS * g + 16 * h;
-}
-
 // Team reduction through LDS + the leader's check.  Returns true for the wave
 // that has to store.  Every wave of the workgroup must call this once.  The
 // accumulators are NT vectors of EV floats per lane (2 x 16 for the 32x32x16
@@ -457,48 +449,6 @@ __device__ __forceinline__ bool team_reduce(V (&acc)[NT], const SchedEntry &e, i
         }
     }
     return leader;
-}
-
-// Split groups: every part parks its fp32 partial tile in the workspace and bumps
-// the group's counter; the part that arrives last adds the tiles up in part order
-// (so the sum does not depend on arrival order), resets the counter and returns
-// true: it stores the result.  Publication follows the release / acquire pattern
-// of split_publish / split_consume (bsa_device.hpp).
-struct SplitWorkspace {
-    int *counters;     // [batches][strips][split_groups], zero between launches
-    float *tiles;      // [batches][strips][tile_slots][2048]
-    int tile_slots, split_groups;
-};
-
-template <class V, int NT, int EV>
-__device__ __forceinline__ bool split_combine(V (&acc)[NT], const SchedEntry &e, const SchedGroup &sg,
-                                              const SplitWorkspace &ws, int batch)
-{
-    const int l = lane_id();
-    const int parts = e.parts();
-    const size_t cell = (size_t)batch * gridDim.y + blockIdx.y;
-    float *tile0 = ws.tiles + (cell * ws.tile_slots + sg.tile_slot) * 2048;
-    float *mine = tile0 + (size_t)e.part() * 2048;
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int v = 0; v < EV; ++v) park_store(mine + (t * EV + v) * WAVE + l, acc[t][v]);
-    int *counter = ws.counters + cell * ws.split_groups + sg.split_index;
-    if (split_publish(counter) != parts - 1) return false;
-    split_consume();
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int v = 0; v < EV; ++v) acc[t][v] = 0.f;
-    for (int p = 0; p < parts; ++p) {
-        const float *src = tile0 + (size_t)p * 2048;
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-#pragma unroll
-            for (int v = 0; v < EV; ++v) acc[t][v] += park_load(src + (t * EV + v) * WAVE + l);
-    }
-    split_reset(counter);
-    return true;
 }
 
 // FULL: the dense dimension is a multiple of 64, every strip has both 32-wide halves: no per-lane
