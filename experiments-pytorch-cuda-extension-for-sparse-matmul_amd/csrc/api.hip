@@ -309,6 +309,7 @@ int bsa_run_schedule_build(const int32_t *row_blocks, const int32_t *row_offsets
     if (sched_bytes < bsa_run_schedule_bytes(mask_rows, nnz))
         return fail(BSA_ERR_INVALID, "%s: the schedule needs %lld bytes, got %lld", who,
                     (long long)bsa_run_schedule_bytes(mask_rows, nnz), (long long)sched_bytes);
+    if (target_pairs > (nnz > 0 ? nnz : 1)) target_pairs = nnz > 0 ? nnz : 1;    // one run at most: no sum in the build overflows
     return check_launch(bsa::launch_run_schedule_build(row_blocks, row_offsets, mask_rows, nnz, target_pairs, max_strips,
                                                        sched, counts_out, (hipStream_t)stream), who);
 }

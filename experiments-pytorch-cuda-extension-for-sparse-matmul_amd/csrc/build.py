@@ -12,6 +12,13 @@ SOURCES = ["api.hip", "layout_build.hip", "matmul.hip", "dsd_runs.hip", "softmax
 HEADERS = ["bench_yardstick.hip", "bsa_device.hpp", "lds_tiles.hpp", "lds_index_math.hpp", "bsa_internal.hpp", "group_walk.hpp", os.path.join("..", "..", "include", "bsa.h")]
 LIB = os.path.join(HERE, "libbsa_hip.so")
 
+# The same library built with the compile-time alternative of a hand-rolled sequence, for the test that pins the
+# default against it (tests/test_gpu_build_variants.py): full agent-scope fences around the counter of split
+# groups instead of atomic accesses + a wait.
+CHECK_VARIANTS = {
+    "fences": (os.path.join(HERE, "libbsa_hip_fences.so"), ["-DBSA_SPLIT_MODE=1"]),
+}
+
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-fno-gpu-rdc", "-Wall", "-Wno-unused-function",
@@ -21,7 +28,7 @@ FLAGS = [
 
 
 def out_of_date() -> bool:
-    if not os.path.exists(LIB):
+    if not os.path.exists(LIB) or not all(os.path.exists(path) for path, _ in CHECK_VARIANTS.values()):
         return True
     t = os.path.getmtime(LIB)
     return any(os.path.getmtime(os.path.join(HERE, f)) > t for f in SOURCES + HEADERS + ["build.py"])
@@ -63,6 +70,8 @@ def build(force: bool = False, verbose: bool = False, extra_flags=(), lib: str =
     if lib == LIB:
         build_index_host(verbose)
         build_bench_yardstick(verbose)
+        for _, (path, flags) in CHECK_VARIANTS.items():
+            build(force=True, verbose=verbose, extra_flags=flags, lib=path)
     return lib
 
 

@@ -33,7 +33,9 @@ struct RunRecord {
     int row0, row1;       // block rows [row0, row1)
     int p0, p1;           // their pairs in the row table
     int n_cols;           // distinct block columns = strips the run keeps in LDS
-    int pad[3];
+    int table_rows;       // the table the schedule was cut from: its groups ...
+    int table_nnz;        // ... and pairs (the walk leaves without a result when they are not its own)
+    int pad;
     unsigned short cols[64];   // the first n_cols: block column of slot s; the rest repeat the last one
 };
 static_assert(sizeof(RunRecord) == RUN_RECORD_BYTES, "the host sizes the schedule with RUN_RECORD_BYTES");
@@ -59,7 +61,9 @@ __global__ __launch_bounds__(64) void run_schedule_build_kernel(
             r->p0 = run_p0;
             r->p1 = p1;
             r->n_cols = n_cur;
-            r->pad[0] = r->pad[1] = r->pad[2] = 0;
+            r->table_rows = rows;
+            r->table_nnz = nnz;
+            r->pad = 0;
         }
         r->cols[l] = (unsigned short)(n_cur > 0 ? cur[l < n_cur ? l : n_cur - 1] : 0);
         widest = n_cur > widest ? n_cur : widest;
@@ -127,7 +131,6 @@ hipError_t launch_run_schedule_build(const int32_t *row_blocks, const int32_t *r
 }
 
 // ---- the walk ---------------------------------------------------------------------------------------
-constexpr int RUN_STRIPS_PER_WAVE = 4;
 #ifndef BSA_RUN_DEPTH
 #define BSA_RUN_DEPTH 3
 #endif
@@ -159,7 +162,7 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
     const half_t *sp, const half_t *dn, half_t *__restrict__ out,
     const BlockDesc *__restrict__ blocks, const int *__restrict__ offsets,
     const RunRecord *__restrict__ runs, const unsigned char *__restrict__ pair_byte,
-    int n_runs, int batches, int nnz, int DN, int KT, int XT, int sp_shared, int info_off, int box_off)
+    int n_runs, int batches, int nnz, int DN, int KT, int XT, int sp_shared, int info_off, int box_off, int strips)
 {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int batch, ri;
@@ -171,6 +174,11 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
     const int my_col = (int)rec->cols[l];
     const int row0 = rec->row0, row1 = rec->row1, p0 = rec->p0, p1 = rec->p1, n_cols = rec->n_cols;
     const int n = p1 - p0;
+    // A schedule of another table, or a launch sized for another schedule (fewer LDS slots or waves than this run
+    // needs), would index LDS and the operands out of range: the workgroup leaves instead, its rows unwritten.
+    if (rec->table_rows * BS != XT || rec->table_nnz != nnz || n_cols > strips || n_cols < 0 || n < 0 || n > 64 * W ||
+        row0 < 0 || row1 > rec->table_rows || p0 < 0 || p1 > nnz)
+        return;
     int *info = reinterpret_cast<int *>(lds_raw + info_off);
     const int y0 = 64 * (int)blockIdx.y;
     const int g = l >> 4, i = l & 15;
@@ -259,7 +267,7 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
         f4v acc[8] = {{0}, {0}, {0}, {0}, {0}, {0}, {0}, {0}};
         f4v acc_head[8];          // the end of a row begun in an earlier wave, kept until that wave can take it
         bool have_head = false;
-        auto store_group = [&](int group, bool in_loop) {
+        auto store_group = [&](int group) {
 #pragma unroll
             for (int xh = 0; xh < 2; ++xh) {
                 half_t *orow = ob + (size_t)(BS * group + 16 * xh + i) * DN;
@@ -271,8 +279,7 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
                         o[v] = narrow_16<BF>(acc[4 * xh + 2 * u][v]);
                         o[4 + v] = narrow_16<BF>(acc[4 * xh + 2 * u + 1][v]);
                     }
-                    if (in_loop) stg16_uncounted(orow + 32 * u, __builtin_bit_cast(uint4, o));
-                    else stg16(orow + 32 * u, __builtin_bit_cast(uint4, o));
+                    stg16(orow + 32 * u, __builtin_bit_cast(uint4, o));
                 }
             }
         };
@@ -290,7 +297,7 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
                         for (int t = 0; t < 8; ++t) acc_head[t] = acc[t];
                         have_head = true;
                     } else {
-                        store_group(cur, true);
+                        store_group(cur);
                     }
 #pragma unroll
                     for (int t = 0; t < 8; ++t) acc[t] = f4v{0};
@@ -331,7 +338,7 @@ __global__ __launch_bounds__(64 * MAXW) void dsd_runs_f16_kernel(
                 if (iv & 1) mailbox_add(acc, reinterpret_cast<const float *>(lds_raw + box_off + (size_t)v * 8192));
                 if (iv & 4) break;
             }
-            store_group(cur, false);
+            store_group(cur);
         }
     }
     // rows without blocks: zeros
@@ -370,7 +377,7 @@ static hipError_t launch_runs(Kernel kernel, const RunsArgs &p, hipStream_t st)
     const unsigned char *pair_byte = reinterpret_cast<const unsigned char *>(p.sched) + (size_t)p.mask_rows * sizeof(RunRecord);
     kernel<<<grid, block, lds, st>>>((const half_t *)p.a, (const half_t *)p.b, (half_t *)p.c, (const BlockDesc *)p.blocks,
                                      p.offsets, runs, pair_byte, p.n_runs, p.batches, p.nnz, p.N, 32 * p.mask_cols,
-                                     32 * p.mask_rows, p.sparse_shared ? 1 : 0, info_off, box_off);
+                                     32 * p.mask_rows, p.sparse_shared ? 1 : 0, info_off, box_off, p.strips);
     return hipGetLastError();
 }
 

@@ -16,26 +16,6 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-// A 16-byte store the compiler does not see as a memory instruction, for the store of a finished group
-// between two blocks of a pipelined walk: behind a store under a condition the compiler would wait for
-// every load in flight, which cancels the prefetch.  The hardware reads the data registers when the
-// store issues and a wave does not end before its stores are acknowledged; a wave's memory instructions
-// retire in order, so a store the compiler did not count only makes its later waits stricter.  Two rules
-// the compiler would otherwise keep for us: a store of more than 8 bytes is followed by wait states
-// before its data registers are overwritten (the s_nop), and the data and address registers must be
-// results of VALU instructions (conversions, address arithmetic), never of an MFMA directly: a register
-// written by the matrix core needs wait states before a memory instruction reads it that nobody inserts
-// here.  -DBSA_PLAIN_STORES builds the walks with ordinary stores instead (same results).
-__device__ __forceinline__ void stg16_uncounted(void *p, uint4 v)
-{
-#ifdef BSA_PLAIN_STORES
-    *reinterpret_cast<uint4 *>(p) = v;
-#else
-    u32x4 w = {v.x, v.y, v.z, v.w};
-    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 2" ::"v"(p), "v"(w) : "memory");
-#endif
-}
-
 template <bool DSD>
 __device__ __forceinline__ size_t gw_out_offset(int g, int y0, int yt, int l, int DN, int XT)
 {

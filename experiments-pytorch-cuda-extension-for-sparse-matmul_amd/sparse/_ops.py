@@ -76,6 +76,7 @@ class Schedule:
         self.waves = waves
         self.cap = cap
         self._workspaces = {}
+        self._captured = {}
         self._spares = {}
         self.last_key = None
 
@@ -100,18 +101,27 @@ class Schedule:
         self.last_key = ("attention_backward", id(columns), batches, head_dim, stream)
         return self._zeroed(self.last_key, need)
 
-    MAX_WORKSPACES = 16      # per schedule; the least recently used one goes first
+    MAX_WORKSPACES = 16      # eager ones per schedule; the least recently used one goes first
 
     def _zeroed(self, key, need):
         """Workspace of ``need`` zero bytes for ``key`` (its last item is the stream).  A buffer must be
         zero before its first launch, and under graph capture nothing can be zeroed (a fill recorded
         there only runs at replay, possibly after another graph has used the buffer): every eager call
-        keeps one zeroed spare per shape ready, which a first use under capture takes."""
+        keeps one zeroed spare per shape ready, which a first use under capture takes.
+
+        A buffer handed out under capture is never dropped: the captured graph holds its raw address and
+        may be replayed at any time.  An eager one is dropped only after the stream it was used on has
+        drained (a launch still in flight parks partial tiles there)."""
         if need == 0:
             return None, 0
-        ws = self._workspaces.pop(key, None)
         capturing = torch.cuda.is_current_stream_capturing()
         spares = self._spares.setdefault(key[:-1], [])
+        ws = self._captured.get(key)
+        if ws is not None:                              # the graph that owns it is being extended or re-captured
+            if not capturing and not spares:
+                spares.append(torch.zeros(need, dtype=torch.uint8, device=self.table.device))
+            return ws, need
+        ws = self._workspaces.pop(key, None)
         if ws is None:
             if capturing:
                 if not spares:
@@ -122,14 +132,24 @@ class Schedule:
                 ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
         if not capturing and not spares:
             spares.append(torch.zeros(need, dtype=torch.uint8, device=self.table.device))
+        if capturing:
+            self._captured[key] = ws
+            return ws, need
         self._workspaces[key] = ws                      # most recently used last
         while len(self._workspaces) > self.MAX_WORKSPACES:
-            self._workspaces.pop(next(iter(self._workspaces)))
+            old_key = next(iter(self._workspaces))
+            self._drain(old_key[-1])
+            self._workspaces.pop(old_key)
         return ws, need
+
+    def _drain(self, stream_handle):
+        """Waits for the stream a workspace was used on before the workspace is given back to the allocator."""
+        torch.cuda.ExternalStream(stream_handle, device=self.table.device).synchronize()
 
     def discard(self, key):
         """Forget the workspace of ``key``: a launch that failed may have left its counters non-zero."""
         self._workspaces.pop(key, None)
+        self._captured.pop(key, None)
 
 
 class RunSchedule:

@@ -56,6 +56,28 @@ def rel_err(out, ref) -> float:
     return float(np.max(np.abs(out - ref))) / (denom if denom > 0 else 1.0)
 
 
+def local_err(out, ref, floor: float = 1e-3) -> float:
+    """Largest error of any output row and of any 32 x 32 output tile, each normalised by its OWN largest
+    reference value (not less than ``floor`` times the global one, so that rows and tiles that are zero
+    or nearly so are held to an absolute bar).  A mistake confined to rows or blocks of small magnitude
+    passes ``rel_err`` and fails here.  Works on dense results ``[..., M, N]`` and on block stacks
+    ``[..., nnz, 32, 32]`` alike (the last two axes are tiled)."""
+    out = np.asarray(out, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    if ref.size == 0:
+        return 0.0
+    top = float(np.max(np.abs(ref)))
+    low = floor * (top if top > 0 else 1.0)
+    diff = np.abs(out - ref)
+    rows = diff.max(axis=-1) / np.maximum(np.abs(ref).max(axis=-1), low)
+    worst = float(rows.max())
+    m, n = ref.shape[-2:]
+    if m % 32 == 0 and n % 32 == 0:
+        tiled = lambda x: x.reshape(x.shape[:-2] + (m // 32, 32, n // 32, 32)).max(axis=(-3, -1))
+        worst = max(worst, float((tiled(diff) / np.maximum(tiled(np.abs(ref)), low)).max()))
+    return worst
+
+
 def operand_shapes(mode, mask, free, trans_a, trans_b, batch=(2,)):
     """Stored shapes of a and b for a product on `mask` with free dense dim `free`."""
     R, C = mask.shape

@@ -345,3 +345,47 @@ def test_run_walk_in_a_hip_graph(small_launches):
         torch.cuda.synchronize()
         assert torch.equal(out, eager), r
         eager = sparse.matmul(a, b, "dsd", L)          # eager work between the replays
+
+
+def test_a_schedule_of_another_table_or_launch_is_left_alone():
+    """The walk indexes LDS and the operands with what the schedule's records hold.  A schedule cut from another
+    table (same number of rows, other pairs), or a launch that reserves fewer strips than a run keeps, must not
+    touch memory: the workgroups leave and the result stays as it was."""
+    import sparse
+    from sparse import kernel as K
+    mask = _attention_mask(24, 3, 4)
+    other = _attention_mask(24, 2, 6)
+    L, L_other = sparse.SparseLayout(torch.as_tensor(mask)), sparse.SparseLayout(torch.as_tensor(other))
+    assert L.num_blocks != L_other.num_blocks
+    rs_other, _, _ = _build(L_other, 30, 32)
+    rs, _, _ = _build(L, 30, 32)
+    g = torch.Generator().manual_seed(9)
+    a = torch.randn(2, L.num_blocks, 32, 32, generator=g).half().cuda()
+    b = torch.randn(2, 32 * 24, 64, generator=g).half().cuda()
+    rc, out = _call(L, rs_other, a, b, 8)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.isnan(out).all()
+    rows = 24
+    out = torch.full((2, 32 * rows, 64), float("nan"), dtype=torch.float16, device="cuda")
+    assert rs.strips > 2
+    rc = K.lib.bsa_matmul_dsd_runs(K.BSA_F16, a.data_ptr(), b.data_ptr(), out.data_ptr(), L.row_layout[0].data_ptr(),
+                                   L.row_layout[1].data_ptr(), rs.table.data_ptr(), rs.runs, 2, rs.pairs, 8, rows, rows,
+                                   L.num_blocks, 2, 2, 64, K.current_stream())      # claims 2 strips per run
+    torch.cuda.synchronize()
+    assert rc == 0
+    written = ~torch.isnan(out).any(-1).any(0).reshape(rows, 32).any(-1)              # block rows with a result
+    assert not written.all()                                                          # the runs that need more left
+    ref = mo.matmul(to_np(a), to_np(b), "dsd", mask).reshape(2, rows, 32, 64)
+    got = to_np(out).reshape(2, rows, 32, 64)
+    for r in range(rows):
+        if written[r]:
+            assert rel_err(got[:, r], ref[:, r]) <= tol_of(torch.float16)
+
+
+def test_a_huge_target_is_one_run():
+    import sparse
+    from sparse import _ops
+    mask = _attention_mask(12, 2, 4)
+    L = sparse.SparseLayout(torch.as_tensor(mask))
+    rs = _ops.RunSchedule(L.row_layout[0], L.row_layout[1], 2 ** 31 - 1, 39)
+    assert rs.runs == 1 and rs.pairs == L.num_blocks

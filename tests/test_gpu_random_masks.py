@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import attention_oracle as ao, matmul_oracle as mo, softmax_oracle as so
-from helpers import operand_shapes, rel_err, to_np
+from helpers import local_err, operand_shapes, rel_err, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -46,6 +46,7 @@ def test_matmul_modes(name, mask):
         assert tuple(c.shape) == ref.shape
         if ref.size:
             assert rel_err(to_np(c), ref) <= 2e-3, (mode, ta, tb, free, batch)
+            assert local_err(to_np(c), ref) <= 2e-3, (mode, ta, tb, free, batch)
 
 
 @pytest.mark.parametrize("name,mask", MASKS, ids=[n for n, _ in MASKS])
