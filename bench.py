@@ -24,6 +24,7 @@ runs, the fastest and slowest are reported beside it.  A streaming copy of the s
 that moves nothing are timed beside it (`read_us`, `write_us`, `empty_launch_us`).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--sets S] [--no-cpu] [--no-attention] [--no-dense] [--no-configs]
+    python bench.py --traffic-from FETCH_CSV WRITE_CSV      (summarises two counter runs, see profiles/)
 """
 import argparse
 import json
@@ -36,6 +37,66 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
+
+
+def kernel_sources_sha256() -> str:
+    """One hash over the sources libbsa_hip.so is built from (csrc/build.py lists them)."""
+    import hashlib
+    csrc = os.path.join(ROOT, "experiments-pytorch-cuda-extension-for-sparse-matmul_amd", "csrc")
+    sys.path.insert(0, csrc)
+    import build as csrc_build
+    h = hashlib.sha256()
+    for name in sorted(csrc_build.SOURCES + [x for x in csrc_build.HEADERS if x.endswith(".hpp")]):
+        with open(os.path.join(csrc, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
+# kernel name fragment -> row of the traffic table (rocprofv3 --pmc, one counter per run)
+TRAFFIC_KERNELS = [("sdd_f16_kernel", "sdd"), ("dsd_runs_f16_kernel", "dsd"), ("gw_f16_kernel", "dds"),
+                   ("softmax_fwd_kernel", "softmax"), ("attention_fwd", "attn"), ("attention_bwd_scores", "bwd_rows"),
+                   ("attention_bwd_dkdv", "bwd_cols")]
+CALIBRATION_KIB = 65536.0          # what the cold 64 MiB torch.neg in front of the timed loops reads, and writes
+
+
+def summarise_traffic(fetch_csv: str, write_csv: str) -> None:
+    """Turns the counter_collection.csv of a FETCH_SIZE run and of a WRITE_SIZE run of this script into
+    profiles/bench_seq4096_hbm_traffic.json: bytes per launch of every kernel, each counter scaled by what it
+    reads for the calibration kernel of known size, stamped with the kernel sources they were measured on."""
+    import collections
+    import csv
+
+    def averages(path, counter):
+        acc = collections.defaultdict(list)
+        for row in csv.DictReader(open(path)):
+            if row["Counter_Name"] != counter:
+                continue
+            name = row["Kernel_Name"]
+            if "neg" in name and int(row.get("Grid_Size", "0")) >= (16 << 20) // 4:
+                acc["calibration"].append(float(row["Counter_Value"]))
+            for frag, op in TRAFFIC_KERNELS:
+                if frag in name:
+                    acc[op].append(float(row["Counter_Value"]))
+                    break
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+    fetch, write = averages(fetch_csv, "FETCH_SIZE"), averages(write_csv, "WRITE_SIZE")
+    fetch_scale = CALIBRATION_KIB / fetch["calibration"]
+    write_scale = CALIBRATION_KIB / write["calibration"]
+    traffic = {op: int(round(1024 * (fetch[op] * fetch_scale + write.get(op, 0.0) * write_scale)))
+               for _, op in TRAFFIC_KERNELS if op in fetch}
+    out = {"workload": "seq4096_block32_causal-local4-stride8_nnz1530_bh16_d64", "unit": "bytes per launch",
+           "fetch_scale": round(fetch_scale, 4), "write_scale": round(write_scale, 4),
+           "kernel_sources_sha256": kernel_sources_sha256(), "traffic": traffic}
+    with open(os.path.join(ROOT, "profiles", "bench_seq4096_hbm_traffic.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    print("kernel    FETCH_SIZE raw   scaled MB   WRITE_SIZE raw   scaled MB   total MB")
+    for _, op in TRAFFIC_KERNELS:
+        if op in fetch:
+            print(f"{op:9s} {fetch[op]:12.1f} {fetch[op] * fetch_scale * 1024 / 1e6:11.2f} {write.get(op, 0.0):16.1f} "
+                  f"{write.get(op, 0.0) * write_scale * 1024 / 1e6:11.2f} {traffic[op] / 1e6:10.2f}")
+    print(f"calibration: FETCH_SIZE {fetch['calibration']:.1f}, WRITE_SIZE {write['calibration']:.1f} KiB for "
+          f"{CALIBRATION_KIB:.0f} KiB each way: scale factors {fetch_scale:.3f}, {write_scale:.3f}")
 
 
 def main():
@@ -53,7 +114,13 @@ def main():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense torch.matmul yardstick")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: summarise two rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE) into "
+                         "profiles/bench_seq4096_hbm_traffic.json")
     args = ap.parse_args()
+    if args.traffic_from:
+        summarise_traffic(*args.traffic_from)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; the path shards over batch*heads with no "
                  "communication, so --gpus N > 1 is not implemented.")
@@ -449,11 +516,14 @@ def main():
         del c5, sc5, p5
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/): same
-    # workload, same kernels; absent file -> null
+    # workload, same kernels.  The file names the kernel sources it was measured on; when they have
+    # changed since (or the file is absent) the figure is stale and null is reported instead.
     traffic = {}
     try:
         with open(os.path.join(ROOT, "profiles", "bench_seq4096_hbm_traffic.json")) as f:
-            traffic = json.load(f)["traffic"]
+            measured = json.load(f)
+        if measured.get("kernel_sources_sha256") == kernel_sources_sha256():
+            traffic = measured["traffic"]
     except (OSError, ValueError, KeyError):
         pass
     for name in per_op:
