@@ -20,8 +20,9 @@ The K timed steps are run `--repeats` times (default 7); `ms_per_step` / `value`
 runs, the fastest and slowest are reported beside it.  A streaming copy of the softmax's byte count
 (non-temporal 16-byte loads and stores, csrc/bench_yardstick.hip) is timed the same way in the same run:
 `yardstick` says what a plain copy reaches on this box in this minute, and every kernel carries
-`vs_copy` = its algorithmic GB/s over the copy's.  The same bytes as a read alone, as a write alone, and a launch
-that moves nothing are timed beside it (`read_us`, `write_us`, `empty_launch_us`).
+`vs_copy` = its algorithmic GB/s over the copy's.  `torch.Tensor.copy_` over the same buffers (`torch_copy_us`,
+`vs_torch_copy`) is the same yardstick from a kernel that is not this repository's.  The same bytes as a read
+alone, as a write alone, and a launch that moves nothing are timed beside it (`read_us`, `write_us`, `empty_launch_us`).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--sets S] [--no-cpu] [--no-attention] [--no-dense] [--no-configs]
     python bench.py --traffic-from FETCH_CSV WRITE_CSV      (summarises two counter runs, see profiles/)
@@ -251,6 +252,17 @@ def main():
     copy_gbs = 2 * copy_bytes / (copy_ms * 1e-3) / 1e9
     yardstick = {"what": "non-temporal copy, 16 B per lane, 4 loads in flight", "bytes_in": copy_bytes, "bytes_out": copy_bytes,
                  "us": round(copy_ms * 1e3, 3), "GBps": round(copy_gbs, 1), "hbm_frac": round(copy_gbs / HBM_PEAK_GBS, 4)}
+    # an independent yardstick: the same bytes moved by torch's own device-to-device copy (not a kernel of this
+    # repository), in the same graph harness over the same rotating buffers
+    def torch_copy_fn(w):
+        i = next(k for k, v in enumerate(sets) if v is w)
+        copy_dst[i].copy_(w["scores"])
+        return copy_dst[i]
+
+    tc_ms = timed(make_runner(torch_copy_fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+    yardstick["torch_copy_us"] = round(tc_ms * 1e3, 3)
+    yardstick["torch_copy_GBps"] = round(2 * copy_bytes / (tc_ms * 1e-3) / 1e9, 1)
+    yardstick["torch_copy_hbm_frac"] = round(2 * copy_bytes / (tc_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
     # the same stream as a read alone and as a write alone, and a launch that moves nothing: what the hardware
     # does with 50 MB in one direction, and what a launch costs before its first byte
     bench_lib.bsa_bench_read_nt.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
@@ -282,7 +294,8 @@ def main():
         ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
         gbs = bytes_alg[name] / (ms * 1e-3) / 1e9
         per_op[name] = {"us": round(ms * 1e3, 3), "GBps": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
-                        "vs_copy": round(gbs / copy_gbs, 3), "algorithmic_MB": round(bytes_alg[name] / 1e6, 3)}
+                        "vs_copy": round(gbs / copy_gbs, 3), "vs_torch_copy": round(gbs / yardstick["torch_copy_GBps"], 3),
+                        "algorithmic_MB": round(bytes_alg[name] / 1e6, 3)}
         if name != "softmax":
             tf = flops_one / (ms * 1e-3) / 1e12
             per_op[name]["nnz_TFLOPs"] = round(tf, 2)

@@ -1055,15 +1055,23 @@ static hipError_t launch_sdd_f32(const MatmulArgs &p, hipStream_t st)
                      sched_slots(p), p.sched_wgs, p.batches, p.nnz, p.M, p.N, p.K
     const int kbs = p.K / BS;
     const size_t lds = (size_t)p.sched_waves * kbs * F32_TILE_BYTES;
-    if (kbs <= 4 && lds <= 65536) {
+    if (kbs <= 4 && lds <= 163840) {      // at most 8 waves x 4 tiles of 4864 bytes: a compute unit's 160 KB hold it
+        auto launch = [&](auto kernel) {
+            hipError_t err = hipSuccess;
+            if (lds > 65536)
+                err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (err != hipSuccess) return err;
+            kernel<<<grid, block, lds, st>>>(BSA_SDD_ARGS);
+            return hipGetLastError();
+        };
         switch (kbs) {
-            case 1: sdd_f32_tiled_kernel<A_KC, B_KC, 1><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
-            case 2: sdd_f32_tiled_kernel<A_KC, B_KC, 2><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
-            case 3: sdd_f32_tiled_kernel<A_KC, B_KC, 3><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
-            default: sdd_f32_tiled_kernel<A_KC, B_KC, 4><<<grid, block, lds, st>>>(BSA_SDD_ARGS); break;
+            case 1: return launch(sdd_f32_tiled_kernel<A_KC, B_KC, 1>);
+            case 2: return launch(sdd_f32_tiled_kernel<A_KC, B_KC, 2>);
+            case 3: return launch(sdd_f32_tiled_kernel<A_KC, B_KC, 3>);
+            default: return launch(sdd_f32_tiled_kernel<A_KC, B_KC, 4>);
         }
-    } else
-        sdd_f32_kernel<A_KC, B_KC><<<grid, block, 0, st>>>(BSA_SDD_ARGS);
+    }
+    sdd_f32_kernel<A_KC, B_KC><<<grid, block, 0, st>>>(BSA_SDD_ARGS);
 #undef BSA_SDD_ARGS
     return hipGetLastError();
 }
@@ -1176,16 +1184,24 @@ constexpr int MAX_DEVICES = 64;
 std::mutex g_scratch_mutex;
 void *g_scratch_ptr[MAX_DEVICES] = {nullptr};
 
-hipError_t static_scratch(void **ptr)
+// The array of the device that holds `on_device` (the result of the call): each GPU has its own copy, and the
+// caller's current device need not be the one its pointers live on.
+hipError_t static_scratch(const void *on_device, void **ptr)
 {
-    int dev = -1;
-    hipError_t err = hipGetDevice(&dev);
+    hipPointerAttribute_t attr;
+    hipError_t err = hipPointerGetAttributes(&attr, on_device);
     if (err != hipSuccess) return err;
+    const int dev = attr.device;
     if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
+        int current = -1;
+        err = hipGetDevice(&current);
+        if (err != hipSuccess) return err;
+        if (current != dev && (err = hipSetDevice(dev)) != hipSuccess) return err;
         void *p = nullptr;
         err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (current != dev) (void)hipSetDevice(current);
         if (err != hipSuccess) return err;
         g_scratch_ptr[dev] = p;
     }
@@ -1209,7 +1225,7 @@ hipError_t launch_group_walk_static_scratch(int dtype, bool dsd, const MatmulArg
     if (need > (size_t)BSA_STATIC_SCRATCH_BYTES) return hipErrorOutOfMemory;   // the C ABI checks first and says why
     if (need > 0) {
         void *base = nullptr;
-        hipError_t err = static_scratch(&base);
+        hipError_t err = static_scratch(p.c, &base);
         if (err != hipSuccess) return err;
         // the counters must start at zero and the buffer keeps what the last call left (an earlier launch
         // may have failed midway); a kernel clears them, so that the call can sit in a captured graph

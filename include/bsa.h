@@ -186,7 +186,9 @@ int bsa_matmul(int mode, int dtype, const void *a, const void *b, void *c,
  * counters it uses with a small kernel on `stream` before the walk, so the state a previous
  * call left behind does not matter.  All calls on one GPU share the buffer: calls that may
  * overlap in time on one GPU (different streams, different threads) race and must be
- * serialised by the caller.
+ * serialised by the caller.  The buffer used is that of the GPU the result `c` lives on,
+ * whatever the caller's current device.  The first call on a GPU looks the buffer's address
+ * up (hipGetSymbolAddress): make it outside graph capture.
  */
 #define BSA_STATIC_SCRATCH_BYTES (16u << 20)
 int bsa_matmul_noalloc(int mode, int dtype, const void *a, const void *b, void *c,

@@ -132,3 +132,50 @@ def test_noalloc_refuses_more_scratch_than_it_has():
                                   blocks.numel() // 2, batches, batches, case["M"], case["N"], case["K"], 0, 0,
                                   k.current_stream())
     assert rc == -3 and b"static buffer" in k.lib.bsa_last_error()
+
+
+def test_noalloc_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point is for.  After one eager call on the device (which looks up the scratch array's
+    address), a call with split groups is captured on a side stream and replayed; between the replays an eager
+    call of another shape uses, and dirties, the same scratch.  Every replay must give bsa_matmul's bits, and the
+    device allocator must hold exactly what it held before."""
+    from sparse import kernel as k
+    case, ref = _case("dds", False, False, ZOO["long_col_70x3"], 128, 2, torch.float16, 7, (2, 2))
+    other, _ = _case("dsd", False, False, ZOO["long_row_5x40"], 64, 3, torch.float16, 8, (3, 2))
+    assert case["sched"].split_groups > 0 and other["sched"].split_groups > 0
+    s = case["sched"]
+    need = k.lib.bsa_matmul_workspace_bytes(k.BSA_DDS, s.tile_slots, s.split_groups, case["batches"], case["M"], case["N"])
+    want = _call("bsa_matmul", workspace=torch.zeros(need, dtype=torch.uint8, device="cuda"), **case)
+    _call("bsa_matmul_noalloc", workspace=None, **other)          # first call on this device: outside capture
+    torch.cuda.synchronize()
+
+    out = torch.empty_like(want)
+    head = (k.BSA_DDS, k.BSA_F16, case["a"].data_ptr(), case["b"].data_ptr(), out.data_ptr(),
+            case["layout"].col_layout[0].data_ptr(), case["layout"].col_layout[1].data_ptr(),
+            case["layout"].col_layout[1].numel() - 1, s.table.data_ptr(), s.workgroups, s.waves, s.tile_slots, s.split_groups)
+    tail = (case["layout"].row_layout[1].numel() - 1, case["layout"].col_layout[1].numel() - 1,
+            case["layout"].col_layout[0].numel() // 2, case["batches"], case["batches"], case["M"], case["N"], case["K"], 0, 0)
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
+    k.check(k.lib.bsa_matmul_noalloc(*head, *tail, k.current_stream()))
+    torch.cuda.synchronize()
+    after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
+    assert after == before, (before, after)
+    assert torch.equal(out, want)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        out.fill_(float("nan"))
+        with torch.cuda.graph(graph, stream=side):
+            k.check(k.lib.bsa_matmul_noalloc(*head, *tail, k.current_stream()))
+    for replay in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+        _call("bsa_matmul_noalloc", workspace=None, **other)      # the same scratch, another shape, in between
+        torch.cuda.synchronize()
+    assert rel_err(to_np(out), ref) <= tol_of(torch.float16)
