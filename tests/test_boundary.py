@@ -170,7 +170,7 @@ def test_workspace_is_never_created_under_graph_capture(monkeypatch):
     import torch
     from sparse import _ops
     sched = object.__new__(_ops.Schedule)
-    sched._workspaces, sched._spares = {}, {}
+    sched._workspaces, sched._captured, sched._spares = {}, {}, {}
     assert sched._zeroed(("attention", 2, 64, 7), 0) == (None, 0)
     monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
     with pytest.raises(RuntimeError, match="eagerly"):
