@@ -490,7 +490,21 @@ def main():
             run_config(f"seq4096_{name}_fp32", fn, 2 * len(sets32), flops=flops_one, nbytes=b32)
             configs[f"seq4096_{name}_fp32"]["mfma_f32_frac"] = round(
                 configs[f"seq4096_{name}_fp32"]["nnz_TFLOPs"] / 157.3, 4)
-        del sets32
+        # SDD in fp32 at head dim 128 (four k-blocks: the widest the tiled kernel keeps resident, 78 KB of LDS per
+        # workgroup with the package's schedule)
+        g128 = torch.Generator().manual_seed(1128)
+        qk128 = [(torch.randn(B, seq, 128, generator=g128).to(dev), torch.randn(B, seq, 128, generator=g128).to(dev))
+                 for _ in range(2)]
+        turn128 = [0]
+
+        def sdd128():
+            turn128[0] += 1
+            q128, k128 = qk128[turn128[0] % 2]
+            return sparse.matmul(q128, k128, "sdd", layout, False, True)
+
+        run_config("seq4096_sdd_fp32_k128", sdd128, 4, flops=2 * flops_one, nbytes=(nnz * 1024 + 2 * seq * 128) * B * 4)
+        configs["seq4096_sdd_fp32_k128"]["mfma_f32_frac"] = round(configs["seq4096_sdd_fp32_k128"]["nnz_TFLOPs"] / 157.3, 4)
+        del sets32, qk128
         c5 = on_gpu(wl.config5())
         l5 = sparse.SparseLayout(c5["mask"])
         n5, b5 = l5.num_blocks, 48
