@@ -288,14 +288,20 @@ def main():
             yardstick[key + "_GBps"] = round(copy_bytes / (ms * 1e-3) / 1e9, 1)
     del copy_dst
 
-    # per-kernel average launch duration: REPS launches per graph, events around the replays
+    # per-kernel average launch duration: REPS launches per graph, events around the replays; like the headline,
+    # the median of `--repeats` runs (a launch's time depends on what the last-level cache holds when it starts,
+    # which shifts from run to run), fastest and slowest beside it
     per_op = {}
     for name, fn in ops.items():
-        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+        runners = make_runner(fn, REPS)
+        runs = sorted(timed(runners, max(args.steps // REPS, 8), max(args.warmup // REPS, 2) if r == 0 else 1) / REPS
+                      for r in range(max(args.repeats, 1)))
+        ms = runs[len(runs) // 2]
         gbs = bytes_alg[name] / (ms * 1e-3) / 1e9
         per_op[name] = {"us": round(ms * 1e3, 3), "GBps": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
                         "vs_copy": round(gbs / copy_gbs, 3), "vs_torch_copy": round(gbs / yardstick["torch_copy_GBps"], 3),
-                        "algorithmic_MB": round(bytes_alg[name] / 1e6, 3)}
+                        "algorithmic_MB": round(bytes_alg[name] / 1e6, 3),
+                        "us_min": round(runs[0] * 1e3, 3), "us_max": round(runs[-1] * 1e3, 3)}
         if name != "softmax":
             tf = flops_one / (ms * 1e-3) / 1e12
             per_op[name]["nnz_TFLOPs"] = round(tf, 2)
