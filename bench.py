@@ -11,9 +11,14 @@ A step is one pass of the three products over that batch:
 `value` = nnz-block TFLOP/s = 3 * 2 * nnz * 32 * 32 * 64 * 16 flop / step time.
 The softmax (scale 1/8, causal) is timed in its own loop and reported in GB/s, and the
 attention forward q, k, v -> out as one fused launch next to the chain of three.
-Consecutive launches take the next of several resident operand sets, so every
-launch finds its operands in HBM, not in the 256 MB infinity cache (`--sets 1`
-shows the cache-resident figures).  Launches are replayed
+Consecutive launches take the next of several resident operand sets (`--sets`, default 6), so the
+blocks -- 88 % of a step's bytes, moved with non-temporal loads and stores -- come from and go to HBM on
+every launch.  The dense operands and dense results (42 MB per step, not streamed) are another matter: over
+6 sets they add up to 252 MB and can stay in the 256 MB last-level cache from one replay to the next, over 8
+sets or more they cannot, and the step then takes 57 us instead of 48 (the SDD product, whose only reads
+are q and k, goes from 12.5 to 19.9 us).  `step_regimes` reports the step over 3 sets (dense operands
+cache-resident for certain, as behind the kernel that produced them) and over 16 (every operand from HBM)
+beside the headline; `--sets 1` shows everything cache-resident.  Launches are replayed
 from HIP graphs (the Python call path costs more than a 10 us kernel).
 
 The K timed steps are run `--repeats` times (default 7); `ms_per_step` / `value` are the median of those
@@ -115,6 +120,8 @@ def main():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense torch.matmul yardstick")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    ap.add_argument("--no-regimes", action="store_true",
+                    help="skip the step over 3 and over 16 operand sets (dense operands cache-resident / from HBM)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: summarise two rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE) into "
                          "profiles/bench_seq4096_hbm_traffic.json")
@@ -186,17 +193,18 @@ def main():
 
     stream = torch.cuda.Stream()
 
-    def make_runner(fn, reps=1):
+    def make_runner(fn, reps=1, pool=None):
         """Callables that each run `reps` launches of fn; consecutive launches always take the next
-        operand set, inside a graph as well as from one graph to the next."""
+        operand set of `pool` (default: all of them), inside a graph as well as from one graph to the next."""
+        pool = sets if pool is None else pool
         with torch.cuda.stream(stream), torch.no_grad():
-            for w in sets:
+            for w in pool:
                 fn(w)                          # build schedules / workspaces outside capture
             stream.synchronize()
-        n_graphs = len(sets) if reps % len(sets) else 1
+        n_graphs = len(pool) if reps % len(pool) else 1
         runners = []
         for gi in range(n_graphs):
-            order = [sets[(gi * reps + i) % len(sets)] for i in range(reps)]
+            order = [pool[(gi * reps + i) % len(pool)] for i in range(reps)]
             if args.no_graph:
                 runners.append(lambda order=order: [fn(w) for w in order])
                 continue
@@ -229,6 +237,29 @@ def main():
                        for r in range(max(args.repeats, 1)))
     step_ms = step_runs[len(step_runs) // 2]
     value = 3 * flops_one / (step_ms * 1e-3) / 1e12
+
+    # The two regimes either side of the default rotation.  Non-temporal streams (the blocks, 88 % of the bytes)
+    # come from and go to HBM whatever the rotation; what does not stream -- per step 25 MB of dense operands
+    # and 17 MB of dense results -- stays in the 256 MB last-level cache from one replay to the next while the
+    # sets together hold less than that (up to 6 sets, and 6 is the edge), as it would behind the kernel that
+    # produced it in a model.  Few sets: dense operands cache-resident for certain; many: everything from HBM.
+    def step_regime(pool):
+        runs = sorted(timed(make_runner(step, per_graph, pool), max(args.steps // per_graph, 1),
+                            -(-args.warmup // per_graph) if r == 0 else 1) / per_graph for r in range(3))
+        ms = runs[len(runs) // 2]
+        return {"operand_sets": len(pool), "ms_per_step": round(ms, 5),
+                "value": round(3 * flops_one / (ms * 1e-3) / 1e12, 2),
+                "dense_MB_per_replay_cycle": round(len(pool) * 5 * seq * D * B * es / 1e6, 1)}
+
+    regimes = {}
+    if not args.no_regimes:
+        regimes["dense_operands_cache_resident"] = step_regime(sets[:3])
+        extra = []
+        for s in range(len(sets), 16):
+            wk = wl.seq4096(batch=B, head_dim=D, seed=1004 + s)
+            extra.append({k: (v.to(dev) if hasattr(v, "to") else v) for k, v in wk.items()})
+        regimes["every_operand_from_hbm"] = step_regime(sets + extra)
+        del extra
 
     # yardstick: a non-temporal streaming copy of the softmax's bytes (50 MB in, 50 MB out), rotating over
     # as many buffer pairs as there are operand sets, from a HIP graph like every kernel below
@@ -575,6 +606,7 @@ def main():
         "config": {"workload": "seq4096_block32_causal-local4-stride8_nnz1530_bh16_d64: SDD(q,k^T)+DSD(p,v)+DDS(dy^T,w) per step",
                    "operand_sets": args.sets, "launch": "eager" if args.no_graph else f"hip-graph replay, {per_graph} steps per graph"},
         "roofline": roofline,
+        "step_regimes": regimes,
         "yardstick": yardstick,
         "softmax": {"GBps": per_op["softmax"]["GBps"], "us": per_op["softmax"]["us"],
                     "roofline": {"bound": "hbm", "achieved": per_op["softmax"]["GBps"], "peak": HBM_PEAK_GBS,
