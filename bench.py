@@ -42,6 +42,11 @@ sys.path.insert(0, os.path.join(ROOT, "experiments-pytorch-cuda-extension-for-sp
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+# The per-kernel loops (not the headline step, whose K and W are the caller's) time at least this many graph
+# replays of 12 launches after at least this many untimed ones: with fewer a kernel's figure moves by 3-5 %
+# from run to run (clocks and caches have not settled after the 3 ms the loop then lasts).
+KERNEL_LOOP_MIN_REPLAYS = 40
+KERNEL_LOOP_MIN_WARMUP = 8
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
 
 
@@ -283,7 +288,7 @@ def main():
         return copy_dst[i]
 
     REPS = 2 * len(sets)
-    copy_ms = timed(make_runner(copy_fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+    copy_ms = timed(make_runner(copy_fn, REPS), max(args.steps // REPS, KERNEL_LOOP_MIN_REPLAYS), max(args.warmup // REPS, KERNEL_LOOP_MIN_WARMUP)) / REPS
     assert torch.equal(copy_dst[0], sets[0]["scores"])
     copy_gbs = 2 * copy_bytes / (copy_ms * 1e-3) / 1e9
     yardstick = {"what": "non-temporal copy, 16 B per lane, 4 loads in flight", "bytes_in": copy_bytes, "bytes_out": copy_bytes,
@@ -295,7 +300,7 @@ def main():
         copy_dst[i].copy_(w["scores"])
         return copy_dst[i]
 
-    tc_ms = timed(make_runner(torch_copy_fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+    tc_ms = timed(make_runner(torch_copy_fn, REPS), max(args.steps // REPS, KERNEL_LOOP_MIN_REPLAYS), max(args.warmup // REPS, KERNEL_LOOP_MIN_WARMUP)) / REPS
     yardstick["torch_copy_us"] = round(tc_ms * 1e3, 3)
     yardstick["torch_copy_GBps"] = round(2 * copy_bytes / (tc_ms * 1e-3) / 1e9, 1)
     yardstick["torch_copy_hbm_frac"] = round(2 * copy_bytes / (tc_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
@@ -318,7 +323,7 @@ def main():
                     ("write", lambda w: checked(bench_lib.bsa_bench_write_nt(copy_dst[index_of(w)].data_ptr(), copy_bytes,
                                                                                torch.cuda.current_stream().cuda_stream))),
                     ("empty_launch", lambda w: checked(bench_lib.bsa_bench_empty(2048, torch.cuda.current_stream().cuda_stream)))):
-        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+        ms = timed(make_runner(fn, REPS), max(args.steps // REPS, KERNEL_LOOP_MIN_REPLAYS), max(args.warmup // REPS, KERNEL_LOOP_MIN_WARMUP)) / REPS
         yardstick[key + "_us"] = round(ms * 1e3, 3)
         if key != "empty_launch":
             yardstick[key + "_GBps"] = round(copy_bytes / (ms * 1e-3) / 1e9, 1)
@@ -330,7 +335,7 @@ def main():
     per_op = {}
     for name, fn in ops.items():
         runners = make_runner(fn, REPS)
-        runs = sorted(timed(runners, max(args.steps // REPS, 8), max(args.warmup // REPS, 2) if r == 0 else 1) / REPS
+        runs = sorted(timed(runners, max(args.steps // REPS, KERNEL_LOOP_MIN_REPLAYS), max(args.warmup // REPS, KERNEL_LOOP_MIN_WARMUP) if r == 0 else 1) / REPS
                       for r in range(max(args.repeats, 1)))
         ms = runs[len(runs) // 2]
         gbs = bytes_alg[name] / (ms * 1e-3) / 1e9
@@ -360,7 +365,7 @@ def main():
             assert err <= 2e-3, f"fused attention differs from the chain: {err}"
         attention = {}
         for name, fn in (("fused", fused), ("chain", chain)):
-            ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+            ms = timed(make_runner(fn, REPS), max(args.steps // REPS, KERNEL_LOOP_MIN_REPLAYS), max(args.warmup // REPS, KERNEL_LOOP_MIN_WARMUP)) / REPS
             attention[name + "_us"] = round(ms * 1e3, 3)
             attention[name + "_nnz_TFLOPs"] = round(2 * flops_one / (ms * 1e-3) / 1e12, 2)
         attention["speedup"] = round(attention["chain_us"] / attention["fused_us"], 2)
@@ -394,7 +399,7 @@ def main():
                 err = ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
                 assert err <= 4e-3, f"attention backward differs from the chain: {err}"
         for name, fn in (("backward_us", backward_fused), ("backward_chain_us", backward_chain)):
-            ms = timed(make_runner(fn, REPS), max(args.steps // REPS, 8), max(args.warmup // REPS, 2)) / REPS
+            ms = timed(make_runner(fn, REPS), max(args.steps // REPS, KERNEL_LOOP_MIN_REPLAYS), max(args.warmup // REPS, KERNEL_LOOP_MIN_WARMUP)) / REPS
             attention[name] = round(ms * 1e3, 3)
 
     def graph_time_us(fn, reps, iters=10):
